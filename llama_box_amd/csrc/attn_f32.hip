@@ -46,6 +46,15 @@ __device__ __forceinline__ float mask_ld(const char * __restrict__ mrow, const i
 // between query and cell: -r1 ln(1 + r2 distance)
 __device__ __forceinline__ float mask_term(const float mv, const bool pen, const float r1, const float r2) { return pen ? -r1 * logf(1.0f + r2 * mv) : mv; }
 
+// the score of a visible cell before the mask's term: dot product x scale x a per-head factor, then optionally soft-capped (cap tanh(. / cap))
+__device__ __forceinline__ float attn_score(const float d, const float scale, const float temp, const float cap) {
+    const float sc = d * scale * temp;
+    return cap > 0.0f ? cap * tanhf(sc / cap) : sc;
+}
+// weights that are no soft-max: sigmoid(score + bias) for every visible cell on its own, nothing normalised over the cells (`sig` = per head a factor on the score,
+// then per head the bias).  The kernels keep their running maximum at 0, rescale by 1 and skip the division by the sum.
+__device__ __forceinline__ float attn_sigmoid(const float z) { return 1.0f / (1.0f + expf(-z)); }
+
 // acc[r] += sum over the block's visible cells of p[cell] * V[cell][lane + 64 r]: no branches around the loads (a lane beyond the row's end re-reads the last
 // column, its sum is dropped later; hidden cells enter with weight 0)
 template <int VT, int CELLS, int RR>
@@ -107,7 +116,7 @@ __device__ __forceinline__ void attn_f32_pv8(const float p, const uint64_t live,
 
 template <int KT, int VT>
 __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const int has_mask, const float * __restrict__ sinks,
-                                                       const float * __restrict__ r12, const tdesc dst, const float scale) {
+                                                       const float * __restrict__ r12, const tdesc dst, const float scale, const float * __restrict__ sig, const float softcap) {
     __shared__ float qs[ATTN_F32_MAX_D];
     __shared__ float part_acc[4][ATTN_F32_MAX_D];
     __shared__ float part_m[4], part_l[4];
@@ -127,8 +136,10 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
     // (value rows of 256 .. 512 two-byte entries: a lane owns eight neighbouring columns)
     const bool v_vec8 = VT != GGML_TYPE_F32 && DV > 256 && DV <= 512 && (DV % 8) == 0 && (v.nb[1] % 16) == 0 && (v.nb[2] % 16) == 0 && (((uintptr_t) v.data) & 15) == 0;
     const bool k_vec = KT != GGML_TYPE_F32 && (DK % 8) == 0 && (k.nb[1] % 16) == 0 && (k.nb[2] % 16) == 0 && (((uintptr_t) k.data) & 15) == 0;
-    float m = ATTN_F32_LOW, l = 0.0f;
-    if (sinks && wave == 0) { m = sinks[h]; l = 1.0f; }  // the sink: exp(sink - m) = 1 in the denominator, nothing in the numerator
+    const bool sgm = sig != nullptr;
+    const float s_temp = sgm ? sig[h] : 1.0f, s_bias = sgm ? sig[q.ne[2] + h] : 0.0f;
+    float m = sgm ? 0.0f : ATTN_F32_LOW, l = 0.0f;
+    if (sinks && wave == 0 && !sgm) { m = sinks[h]; l = 1.0f; }  // the sink: exp(sink - m) = 1 in the denominator, nothing in the numerator
     float acc[ATTN_F32_MAX_D / 64];
 #pragma unroll
     for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) acc[r] = 0.0f;
@@ -161,13 +172,19 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
                 for (int i = 0; i < DK; ++i) d = fmaf(qs[i], kv_ld<KT>(krow, i), d);
             } else
             for (int i = 0; i < DK; ++i) d = fmaf(qs[i], kv_ld<KT>(krow, i), d);
-            s = d * scale + mask_term(mv, pen, r1, r2);
+            s = attn_score(d, scale, s_temp, softcap) + mask_term(mv, pen, r1, r2);
         }
-        const float m_new = fmaxf(m, wave_max_f(s));
-        const float p = vis ? expf(s - m_new) : 0.0f;
-        const float corr = expf(m - m_new);
-        l = l * corr + wave_sum_f(p);
-        m = m_new;
+        float p, corr;
+        if (sgm) {
+            p = vis ? attn_sigmoid(s + s_bias) : 0.0f;
+            corr = 1.0f;
+        } else {
+            const float m_new = fmaxf(m, wave_max_f(s));
+            p = vis ? expf(s - m_new) : 0.0f;
+            corr = expf(m - m_new);
+            l = l * corr + wave_sum_f(p);
+            m = m_new;
+        }
 #pragma unroll
         for (int r = 0; r < ATTN_F32_MAX_D / 64; ++r) acc[r] *= corr;
         // the visible cells' value rows, CELLS at a time with all their loads in flight together: a wave pays one trip to memory per group (measured: 2 us
@@ -196,7 +213,7 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
     for (int w = 1; w < 4; ++w) M = fmaxf(M, part_m[w]);
     float L = 0.0f, cw[4];
     for (int w = 0; w < 4; ++w) { cw[w] = expf(part_m[w] - M); L += part_l[w] * cw[w]; }
-    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+    const float inv = sgm ? 1.0f : (L > 0.0f ? 1.0f / L : 0.0f);
     float * out = (float *) (dst.data + h * dst.nb[1] + t * dst.nb[2]);
     for (int dcol = lane; dcol < DV; dcol += 64) {
         float o = 0.0f;
@@ -208,7 +225,7 @@ __global__ void __launch_bounds__(256) k_attn_f32_rows(const tdesc q, const tdes
 // prompt batches: 64 query tokens x one head per workgroup; K / V blocks of 64 cells staged in LDS as f32
 template <int KT, int VT, int DKP, int DVP>   // DKP / DVP: head sizes rounded up to a multiple of 32 / 64 (LDS row lengths)
 __global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks,
-                                                       const float * __restrict__ r12, const tdesc dst, const float scale) {
+                                                       const float * __restrict__ r12, const tdesc dst, const float scale, const float * __restrict__ sig, const float softcap) {
     constexpr int QT = 64, KB = 64, QW = QT / 4;  // queries per workgroup, cells per block, queries per wave
     constexpr int KS = DKP + 1;                   // K row stride in LDS (odd: lanes that read column i of 64 different rows hit 64 different banks)
     extern __shared__ float lds[];
@@ -230,11 +247,13 @@ __global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdes
         const int64_t t = t0 + qi;
         Qs[e] = (t < n_q && i < DK) ? ((const float *) (q.data + t * q.nb[1] + h * q.nb[2]))[i] : 0.0f;
     }
+    const bool sgm = sig != nullptr;
+    const float s_temp = sgm ? sig[h] : 1.0f, s_bias = sgm ? sig[q.ne[2] + h] : 0.0f;
     float m[QW], l[QW], acc[QW][DVP / 64];
 #pragma unroll
     for (int qi = 0; qi < QW; ++qi) {
-        m[qi] = sinks ? sinks[h] : ATTN_F32_LOW;
-        l[qi] = sinks ? 1.0f : 0.0f;
+        m[qi] = sgm ? 0.0f : (sinks ? sinks[h] : ATTN_F32_LOW);
+        l[qi] = (sinks && !sgm) ? 1.0f : 0.0f;
 #pragma unroll
         for (int r = 0; r < DVP / 64; ++r) acc[qi][r] = 0.0f;
     }
@@ -277,12 +296,18 @@ __global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdes
             const float * qr = Qs + ql * DKP;
             const float * kr = Ks + lane * KS;
             for (int i = 0; i < DK; ++i) d = fmaf(qr[i], kr[i], d);
-            const float s = vis ? d * scale + mask_term(mv, pen, r1, r2) : -INFINITY;
-            const float m_new = fmaxf(m[qi], wave_max_f(s));
-            const float p = vis ? expf(s - m_new) : 0.0f;
-            const float corr = expf(m[qi] - m_new);
-            l[qi] = l[qi] * corr + wave_sum_f(p);
-            m[qi] = m_new;
+            const float s = vis ? attn_score(d, scale, s_temp, softcap) + mask_term(mv, pen, r1, r2) : -INFINITY;
+            float p, corr;
+            if (sgm) {
+                p = vis ? attn_sigmoid(s + s_bias) : 0.0f;
+                corr = 1.0f;
+            } else {
+                const float m_new = fmaxf(m[qi], wave_max_f(s));
+                p = vis ? expf(s - m_new) : 0.0f;
+                corr = expf(m[qi] - m_new);
+                l[qi] = l[qi] * corr + wave_sum_f(p);
+                m[qi] = m_new;
+            }
 #pragma unroll
             for (int r = 0; r < DVP / 64; ++r) acc[qi][r] *= corr;
             uint64_t todo = live;
@@ -299,7 +324,7 @@ __global__ void __launch_bounds__(256) k_attn_f32_tile(const tdesc q, const tdes
     for (int qi = 0; qi < QW; ++qi) {
         const int64_t t = t0 + wave * QW + qi;
         if (t >= n_q) continue;
-        const float inv = l[qi] > 0.0f ? 1.0f / l[qi] : 0.0f;
+        const float inv = sgm ? 1.0f : (l[qi] > 0.0f ? 1.0f / l[qi] : 0.0f);
         float * out = (float *) (dst.data + h * dst.nb[1] + t * dst.nb[2]);
 #pragma unroll
         for (int r = 0; r < DVP / 64; ++r) {
@@ -327,7 +352,7 @@ __device__ __forceinline__ uint32_t att_bf16_bits(const float f) {
 }
 template <int DK16, int DVT>
 __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks, const float * __restrict__ r12, const tdesc dst,
-                                                       const float scale) {
+                                                       const float scale, const float * __restrict__ sig, const float softcap) {
     constexpr int VS = 36;  // V^T row stride in LDS (bf16 elements): 72 bytes keeps the 8-byte reads aligned and spreads the rows over the banks
     __shared__ __attribute__((aligned(16))) uint16_t Vt[DVT * 32 * VS];
     __shared__ int flag[2];
@@ -355,7 +380,9 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
     }
     const bool pen = r12 != nullptr;
     const float r1 = pen ? r12[h] : 0.0f, r2 = pen ? r12[q.ne[2] + h] : 0.0f;
-    float m = sinks ? sinks[h] : ATTN_F32_LOW, l = sinks ? 1.0f : 0.0f;
+    const bool sgm = sig != nullptr;
+    const float s_temp = sgm ? sig[h] : 1.0f, s_bias = sgm ? sig[q.ne[2] + h] : 0.0f;
+    float m = sgm ? 0.0f : (sinks ? sinks[h] : ATTN_F32_LOW), l = (sinks && !sgm) ? 1.0f : 0.0f;
     att_f16v O[DVT];
 #pragma unroll
     for (int dt = 0; dt < DVT; ++dt)
@@ -433,17 +460,18 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
         float mx = ATTN_F32_LOW;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            S[i] = mv[i] > -INFINITY ? S[i] * scale + mask_term(mv[i], pen, r1, r2) : -INFINITY;
+            S[i] = mv[i] > -INFINITY ? attn_score(S[i], scale, s_temp, softcap) + mask_term(mv[i], pen, r1, r2) : -INFINITY;
             mx = fmaxf(mx, S[i]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m, mx);
-        const float corr = expf(m - m_new);
+        const float m_new = sgm ? 0.0f : fmaxf(m, mx);
+        const float corr = sgm ? 1.0f : expf(m - m_new);
         float ps = 0.0f;
         uint32_t hi[8], lo[8];
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
-            const float p0 = expf(S[i] - m_new), p1 = expf(S[i + 1] - m_new);
+            const float p0 = sgm ? (S[i] > -INFINITY ? attn_sigmoid(S[i] + s_bias) : 0.0f) : expf(S[i] - m_new);
+            const float p1 = sgm ? (S[i + 1] > -INFINITY ? attn_sigmoid(S[i + 1] + s_bias) : 0.0f) : expf(S[i + 1] - m_new);
             ps += p0 + p1;
             const uint32_t h0 = att_bf16_bits(p0), h1 = att_bf16_bits(p1);
             hi[i >> 1] = h0 | (h1 << 16);
@@ -471,7 +499,7 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
         }
     }
     if (!q_live) return;
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    const float inv = sgm ? 1.0f : (l > 0.0f ? 1.0f / l : 0.0f);
     float * out = (float *) (dst.data + h * dst.nb[1] + tq * dst.nb[2]);
 #pragma unroll
     for (int dt = 0; dt < DVT; ++dt)
@@ -490,7 +518,7 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16(const tdesc q, const tdes
 // 32-entry value tiles per wave.
 template <int DKQ, int DVQ>
 __global__ void __launch_bounds__(256) k_attn_mma_bf16_wide(const tdesc q, const tdesc k, const tdesc v, const tdesc mask, const float * __restrict__ sinks, const float * __restrict__ r12,
-                                                            const tdesc dst, const float scale) {
+                                                            const tdesc dst, const float scale, const float * __restrict__ sig, const float softcap) {
     constexpr int VS = 36;
     constexpr int DVT = 4 * DVQ;
     __shared__ __attribute__((aligned(16))) uint16_t Vt[DVT * 32 * VS];
@@ -519,7 +547,9 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16_wide(const tdesc q, const
     }
     const bool pen = r12 != nullptr;
     const float r1 = pen ? r12[h] : 0.0f, r2 = pen ? r12[H + h] : 0.0f;
-    float m = sinks ? sinks[h] : ATTN_F32_LOW, l = sinks ? 1.0f : 0.0f;
+    const bool sgm = sig != nullptr;
+    const float s_temp = sgm ? sig[h] : 1.0f, s_bias = sgm ? sig[q.ne[2] + h] : 0.0f;
+    float m = sgm ? 0.0f : (sinks ? sinks[h] : ATTN_F32_LOW), l = (sinks && !sgm) ? 1.0f : 0.0f;
     att_f16v O[DVQ];
 #pragma unroll
     for (int dt = 0; dt < DVQ; ++dt)
@@ -602,17 +632,18 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16_wide(const tdesc q, const
         float mx = ATTN_F32_LOW;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            S[i] = mv[i] > -INFINITY ? S[i] * scale + mask_term(mv[i], pen, r1, r2) : -INFINITY;
+            S[i] = mv[i] > -INFINITY ? attn_score(S[i], scale, s_temp, softcap) + mask_term(mv[i], pen, r1, r2) : -INFINITY;
             mx = fmaxf(mx, S[i]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m, mx);
-        const float corr = expf(m - m_new);
+        const float m_new = sgm ? 0.0f : fmaxf(m, mx);
+        const float corr = sgm ? 1.0f : expf(m - m_new);
         float ps = 0.0f;
         uint32_t hi[8], lo[8];
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
-            const float p0 = expf(S[i] - m_new), p1 = expf(S[i + 1] - m_new);
+            const float p0 = sgm ? (S[i] > -INFINITY ? attn_sigmoid(S[i] + s_bias) : 0.0f) : expf(S[i] - m_new);
+            const float p1 = sgm ? (S[i + 1] > -INFINITY ? attn_sigmoid(S[i + 1] + s_bias) : 0.0f) : expf(S[i + 1] - m_new);
             ps += p0 + p1;
             const uint32_t h0 = att_bf16_bits(p0), h1 = att_bf16_bits(p1);
             hi[i >> 1] = h0 | (h1 << 16);
@@ -640,7 +671,7 @@ __global__ void __launch_bounds__(256) k_attn_mma_bf16_wide(const tdesc q, const
         }
     }
     if (!q_live) return;
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    const float inv = sgm ? 1.0f : (l > 0.0f ? 1.0f / l : 0.0f);
     float * out = (float *) (dst.data + h * dst.nb[1] + tq * dst.nb[2]);
 #pragma unroll
     for (int dt = 0; dt < DVQ; ++dt)
@@ -687,7 +718,8 @@ bool attn_f32_applies(const tdesc & q, const tdesc & k, const tdesc & v, const t
 }
 
 template <int KT, int VT>
-static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const float * r12, const tdesc & dst, float scale) {
+static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const float * r12, const tdesc & dst, float scale,
+                              const float * sig, float softcap) {
     const int64_t n_q = q.ne[1], H = q.ne[2];
     const int DK = (int) q.ne[0], DV = (int) v.ne[0];
     if constexpr (KT == GGML_TYPE_BF16 && VT == GGML_TYPE_BF16) {
@@ -695,7 +727,7 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
         if (mma_on && attn_mma_bf16_wide_ok(q, k, v, mask, dst)) {  // one shared key/value head with wide rows (latent attention): four waves per 32 (token, head) pairs
             const dim3 grid((unsigned) ((n_q * H + 31) / 32));
             const int dkq = ((DK + 15) / 16 + 3) / 4, dvq = ((DV + 31) / 32 + 3) / 4;  // per wave: 16-entry key groups (<= 10), 32-entry value tiles (<= 4)
-#define MI_ATT_WIDE(A, B) hipLaunchKernelGGL((k_attn_mma_bf16_wide<A, B>), grid, dim3(256), 0, s, q, k, v, *mask, sinks, r12, dst, scale)
+#define MI_ATT_WIDE(A, B) hipLaunchKernelGGL((k_attn_mma_bf16_wide<A, B>), grid, dim3(256), 0, s, q, k, v, *mask, sinks, r12, dst, scale, sig, softcap)
             const int a = dkq <= 3 ? 3 : (dkq <= 5 ? 5 : 10), b = dvq <= 1 ? 1 : (dvq <= 2 ? 2 : 4);
             if (a == 3 && b == 1) MI_ATT_WIDE(3, 1); else if (a == 3 && b == 2) MI_ATT_WIDE(3, 2); else if (a == 3) MI_ATT_WIDE(3, 4);
             else if (a == 5 && b == 1) MI_ATT_WIDE(5, 1); else if (a == 5 && b == 2) MI_ATT_WIDE(5, 2); else if (a == 5) MI_ATT_WIDE(5, 4);
@@ -713,7 +745,7 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
             const dim3 grid((unsigned) ((n_q + 32 * nw - 1) / (32 * nw)), (unsigned) H);
             const dim3 block((unsigned) (64 * nw));
             const int dk16 = (DK + 15) / 16, dvt = (DV + 31) / 32;
-#define MI_ATT_MMA(A, B) hipLaunchKernelGGL((k_attn_mma_bf16<A, B>), grid, block, 0, s, q, k, v, *mask, sinks, r12, dst, scale)
+#define MI_ATT_MMA(A, B) hipLaunchKernelGGL((k_attn_mma_bf16<A, B>), grid, block, 0, s, q, k, v, *mask, sinks, r12, dst, scale, sig, softcap)
             const int a = dk16 <= 2 ? 2 : (dk16 <= 4 ? 4 : 8), b = dvt <= 1 ? 1 : (dvt <= 2 ? 2 : 4);
             if (a == 2 && b == 1) MI_ATT_MMA(2, 1); else if (a == 2 && b == 2) MI_ATT_MMA(2, 2); else if (a == 2) MI_ATT_MMA(2, 4);
             else if (a == 4 && b == 1) MI_ATT_MMA(4, 1); else if (a == 4 && b == 2) MI_ATT_MMA(4, 2); else if (a == 4) MI_ATT_MMA(4, 4);
@@ -729,7 +761,7 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
             const size_t lds = ((size_t) 64 * (dkp + 1) + (size_t) 64 * dvp + (size_t) 64 * dkp) * sizeof(float);
             // (more than the 64 KB a kernel gets by default: up to 97 KB of the CU's 160 KB; the attribute is per device and cheap to set again)
             if (lds > 48 * 1024) (void) hipFuncSetAttribute((const void *) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds);
-            hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, q, k, v, *mask, sinks, r12, dst, scale);
+            hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, q, k, v, *mask, sinks, r12, dst, scale, sig, softcap);
         };
         const bool k64 = DK <= 64, v64 = DV <= 64;
         if (k64 && v64) go(k_attn_f32_tile<KT, VT, 64, 64>, 64, 64);
@@ -738,12 +770,13 @@ static void attn_f32_launch_t(hipStream_t s, const tdesc & q, const tdesc & k, c
         else go(k_attn_f32_tile<KT, VT, 128, 128>, 128, 128);
         return;
     }
-    hipLaunchKernelGGL((k_attn_f32_rows<KT, VT>), dim3((unsigned) n_q, (unsigned) H), dim3(256), 0, s, q, k, v, mask ? *mask : q, mask ? 1 : 0, sinks, r12, dst, scale);
+    hipLaunchKernelGGL((k_attn_f32_rows<KT, VT>), dim3((unsigned) n_q, (unsigned) H), dim3(256), 0, s, q, k, v, mask ? *mask : q, mask ? 1 : 0, sinks, r12, dst, scale, sig, softcap);
 }
 
-void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const float * r12, const tdesc & dst, float scale) {
+void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const float * r12, const tdesc & dst, float scale,
+                     const float * sig, float softcap) {
     if (q.ne[1] == 0 || q.ne[2] == 0) return;
-#define MI_ATTN_F32_CASE(KT, VT) if (k.type == KT && v.type == VT) { attn_f32_launch_t<KT, VT>(s, q, k, v, mask, sinks, r12, dst, scale); return; }
+#define MI_ATTN_F32_CASE(KT, VT) if (k.type == KT && v.type == VT) { attn_f32_launch_t<KT, VT>(s, q, k, v, mask, sinks, r12, dst, scale, sig, softcap); return; }
     MI_ATTN_F32_CASE(GGML_TYPE_F32, GGML_TYPE_F32)
     MI_ATTN_F32_CASE(GGML_TYPE_BF16, GGML_TYPE_BF16)
     MI_ATTN_F32_CASE(GGML_TYPE_F16, GGML_TYPE_F16)

@@ -1035,6 +1035,7 @@ static bool op_numbering_matches_host() {
         {GGML_OP_TRANSPOSE, "TRANSPOSE"}, {GGML_OP_GET_ROWS, "GET_ROWS"}, {GGML_OP_SET_ROWS, "SET_ROWS"}, {GGML_OP_SOFT_MAX, "SOFT_MAX"},
         {GGML_OP_ROPE, "ROPE"}, {GGML_OP_FLASH_ATTN_EXT, "FLASH_ATTN_EXT"}, {GGML_OP_UNARY, "UNARY"}, {GGML_OP_GLU, "GLU"},
         {GGML_OP_NORM, "NORM"}, {GGML_OP_SQR, "SQR"}, {GGML_OP_ARGSORT, "ARGSORT"}, {GGML_OP_CONCAT, "CONCAT"},
+        {GGML_OP_SSM_CONV, "SSM_CONV"}, {GGML_OP_RWKV_WKV6, "RWKV_WKV6"}, {GGML_OP_GATED_LINEAR_ATTN, "GATED_LINEAR_ATTN"},
     };
     bool ok = true;
     for (const auto & e : k_expect) {

@@ -65,7 +65,9 @@ static bool fa_f32_route(const ggml_tensor * op) {
     const ggml_tensor * k = op->src[1];
     const ggml_tensor * v = op->src[2];
     const ggml_tensor * m = op->src[3];
-    if (ggml_abi_op_param_f32(op, 1) != 0.0f || ggml_abi_op_param_f32(op, 2) != 0.0f) return false;  // no ALiBi slopes, no soft-capping there
+    if (ggml_abi_op_param_f32(op, 1) != 0.0f || ggml_abi_op_param_f32(op, 2) < 0.0f) return false;  // no ALiBi slopes there (soft-capping: yes)
+    // src[6]: per head a factor on the score and a bias — the weights are sigmoid(score + bias) instead of a soft-max (no sink then)
+    if (op->src[6] && (op->src[6]->type != GGML_TYPE_F32 || !ggml_abi_is_contiguous(op->src[6]) || ggml_abi_nelements(op->src[6]) != 2 * a->ne[2] || op->src[4])) return false;
     if (op->src[4] && (op->src[4]->type != GGML_TYPE_F32 || ggml_abi_nelements(op->src[4]) < a->ne[2])) return false;
     // src[5]: (r1, r2) per head of a logarithmic distance penalty; the F32 mask then holds distances
     if (op->src[5] && (op->src[5]->type != GGML_TYPE_F32 || !ggml_abi_is_contiguous(op->src[5]) || ggml_abi_nelements(op->src[5]) != 2 * a->ne[2] || !m || m->type != GGML_TYPE_F32)) return false;
@@ -87,7 +89,7 @@ static int fa_route(const ggml_tensor * op) {
         (void) wide_k; (void) wide_v;
         if (plain && (f32_mask || odd_shape) && fa_f32_route(op)) return 4;
     }
-    if (op->src[5]) return 0;  // (the distance penalty is a feature of the 32-bit kernels alone)
+    if (op->src[5] || op->src[6]) return 0;  // (the distance penalty and sigmoid weights are features of the 32-bit kernels alone)
     if (k->type == GGML_TYPE_Q8_0 && v->type == GGML_TYPE_Q8_0) {
         // quantised KV cache: served by the lane-parallel kernel (head_dim 128, 1 .. 8 query heads per KV head, no soft-capping / ALiBi)
         const int64_t g = k->ne[2] ? a->ne[2] / k->ne[2] : 0;
@@ -125,6 +127,43 @@ static int rope_exact_freq(const ggml_tensor * n) {
     if (n->op_params[3] == 2 && n->src[2] && !(n->op_params[2] & GGML_ROPE_TYPE_MROPE)) return 2;
     return (n->op_params[3] == 1 && !n->src[2] && !(n->op_params[2] & GGML_ROPE_TYPE_MROPE) && ggml_abi_op_param_f32(n, 6) == 1.0f && ggml_abi_op_param_f32(n, 7) == 0.0f &&
             ggml_abi_op_param_f32(n, 8) == 1.0f) ? 1 : 0;
+}
+
+// the ops over sequence state (seq.hip) in this backend's own operand layout, marked by op_params[3] == MI_SEQ_OP_TAG (ggml's ops of the same numbers, whose
+// batches are equal-length sequences with the states as graph tensors, are not served):
+//   SSM_CONV, op_params (taps, act, mode): mode 0  src (x [C, T], w [taps, C, M], state, hist [hs, T] i32) -> [C, T, M];
+//                                          mode 1  src (x, upd [hs, n_seq] i32, info [4, n_seq] i32) -> the state (a view of it): the sequences' last taps - 1 inputs
+//   RWKV_WKV6, op_params (H): src (r, k, v, w_pre [D H, T], w0 [D H], u [D H], state, tok [T] i32, info) -> [D, H, T]
+//   GATED_LINEAR_ATTN, op_params (kind 1 delta rule / 2 matrix memory, H, G, tag, cap, q scale): src (q, k [DK G, T], v [DV H, T], gates [2 H, T], params [2 H], state, tok, info) -> [DV, H, T]
+static constexpr int32_t MI_SEQ_OP_TAG = 0x5E9;
+static bool seq_op_ok(const ggml_tensor * op) {
+    if (op->op_params[3] != MI_SEQ_OP_TAG || op->type != GGML_TYPE_F32) return false;
+    auto f32c = [](const ggml_tensor * t) { return t && t->type == GGML_TYPE_F32 && ggml_abi_is_contiguous(t); };
+    auto f32rows = [](const ggml_tensor * t) { return t && t->type == GGML_TYPE_F32 && t->nb[0] == 4 && t->ne[2] == 1 && t->ne[3] == 1; };
+    auto i32c = [](const ggml_tensor * t) { return t && t->type == GGML_TYPE_I32 && ggml_abi_is_contiguous(t); };
+    const ggml_tensor * const * src = op->src;
+    if (op->op == GGML_OP_SSM_CONV) {
+        const int taps = op->op_params[0], mode = op->op_params[2];
+        if (taps < 1 || taps > 16 || !f32rows(src[0])) return false;
+        if (mode == 1) return taps >= 2 && i32c(src[1]) && i32c(src[2]) && src[1]->ne[0] >= taps - 1 && src[2]->ne[0] == 4 && src[1]->ne[1] == src[2]->ne[1] && ggml_abi_is_contiguous(op);
+        if (mode != 0 || !f32c(src[1]) || !ggml_abi_is_contiguous(op)) return false;
+        if (src[1]->ne[0] != taps || src[1]->ne[1] != src[0]->ne[0] || op->ne[0] != src[0]->ne[0] || op->ne[1] != src[0]->ne[1] || op->ne[2] != src[1]->ne[2]) return false;
+        return taps == 1 || (f32c(src[2]) && i32c(src[3]) && src[3]->ne[0] >= taps - 1 && src[3]->ne[1] == src[0]->ne[1]);
+    }
+    const bool wkv = op->op == GGML_OP_RWKV_WKV6;
+    const int kind = wkv ? SEQ_WKV6 : op->op_params[0];
+    if (!wkv && kind != SEQ_DELTA && kind != SEQ_MLSTM) return false;
+    const int H = wkv ? op->op_params[0] : op->op_params[1], G = wkv ? H : op->op_params[2];
+    const ggml_tensor * state = src[wkv ? 6 : 5], * tok = src[wkv ? 7 : 6], * info = src[wkv ? 8 : 7];
+    if (H < 1 || G < 1 || H % G || !f32rows(src[0]) || !f32rows(src[1]) || !f32rows(src[2]) || !f32rows(src[3]) || !f32c(src[4]) || !f32c(state) || !i32c(tok) || !i32c(info)) return false;
+    if (wkv && !f32c(src[5])) return false;
+    const int64_t T = src[0]->ne[1];
+    if (src[0]->ne[0] % G || src[2]->ne[0] % H) return false;
+    const int64_t DK = src[0]->ne[0] / G, DV = src[2]->ne[0] / H;
+    if (!seq_recurrence_ok((int) DK, (int) DV) || src[1]->ne[0] != DK * G || src[1]->ne[1] != T || src[2]->ne[1] != T || src[3]->ne[1] != T) return false;
+    if (src[3]->ne[0] != (wkv ? DK * H : 2 * H) || ggml_abi_nelements(src[4]) != (wkv ? DK * H : 2 * H) || (wkv && ggml_abi_nelements(src[5]) != DK * H)) return false;
+    if (ggml_abi_nelements(tok) != T || info->ne[0] != 4 || state->ne[0] != seq_recurrence_state_floats(kind, H, (int) DK, (int) DV)) return false;
+    return op->ne[0] == DV && op->ne[1] == H && op->ne[2] == T && ggml_abi_is_contiguous(op);
 }
 
 bool supports_op(const ggml_tensor * op) {
@@ -169,7 +208,11 @@ bool supports_op(const ggml_tensor * op) {
         case GGML_OP_SQR:
             return is_f32_contig(a) && is_f32_contig(op);
         case GGML_OP_ARGSORT:
+            // op_params[1] > 1: the entries form that many equal groups of neighbours and only the op_params[2] groups with the largest maxima may come first (descending)
+            if (op->op_params[1] > 1 && (op->op_params[0] != 1 || op->op_params[1] > 256 || a->ne[0] % op->op_params[1] != 0 || op->op_params[2] < 1)) return false;
             return a->type == GGML_TYPE_F32 && a->nb[0] == 4 && op->type == GGML_TYPE_I32 && op->nb[0] == 4 && a->ne[0] <= 65536;
+        case GGML_OP_SSM_CONV: case GGML_OP_RWKV_WKV6: case GGML_OP_GATED_LINEAR_ATTN:
+            return seq_op_ok(op);
         case GGML_OP_MUL_MAT_ID: {
             const ggml_tensor * ids = op->src[2];
             if (!a || !b || !ids || b->type != GGML_TYPE_F32 || op->type != GGML_TYPE_F32 || ids->type != GGML_TYPE_I32 || !ggml_abi_is_contiguous(op)) return false;
@@ -1859,6 +1902,119 @@ static int try_fuse_token_shift(exec_state & st, int i) {
 
 // ADD(mat-mul, bias) -> GELU ... [mat-mul] -> ADD(mat-mul, bias) -> MUL(gelu, .): the gated activation with both biases in one launch.  The second mat-mul, when it
 // sits between, is executed early (its result may not occupy memory that is still read).  Returns true when node i is done (the rest is marked)
+// SOFT_MAX(router logits) -> ARGSORT (descending, optionally group-limited) -> VIEW (top k) ... GET_ROWS(scores as [1, n, T], view) -> SCALE: a router whose weights
+// are the chosen scores of a soft-max over ALL experts, in one launch.  GET_ROWS and SCALE sit behind the expert mat-muls in the graph's order and are executed
+// early, which is legal when nothing in between reads or occupies the memory the weights are written to.  Returns the nodes consumed at position i (0: no match)
+static int try_fuse_router_scores(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * sm = g->nodes[i];
+    const ggml_tensor * a = sm->src[0];
+    if (sm->src[1] || sm->src[2] || ggml_abi_op_param_f32(sm, 0) != 1.0f || ggml_abi_op_param_f32(sm, 1) != 0.0f) return 0;
+    int ka = i + 1;  // the sort: the next node that is no view
+    while (ka < g->n_nodes && !st.done[ka] && is_view_op(g->nodes[ka])) ++ka;
+    if (ka >= g->n_nodes || st.done[ka]) return 0;
+    const ggml_tensor * as = g->nodes[ka];
+    if (as->op != GGML_OP_ARGSORT || as->src[0] != sm || as->op_params[0] != 1 || !is_f32_contig(a) || !is_f32_contig(sm) || a->ne[0] > 256 || a->ne[2] != 1 || a->ne[3] != 1 ||
+        !ggml_abi_is_contiguous(as)) return 0;
+    int kg = -1, ks = -1;
+    const int limit = std::min(g->n_nodes, i + 24);
+    for (int k = ka + 1; k < limit && kg < 0; ++k) {
+        const ggml_tensor * t = g->nodes[k];
+        if (!st.done[k] && t->op == GGML_OP_GET_ROWS && t->src[1] && t->src[1]->view_src == as && t->src[1]->view_offs == 0) kg = k;
+    }
+    const ggml_tensor * gr = kg >= 0 ? g->nodes[kg] : nullptr;
+    if (!gr || through_views(gr->src[0]) != sm || gr->src[0]->ne[0] != 1 || gr->src[1]->ne[1] != a->ne[1] || !single_use(st, gr)) return 0;
+    for (int k = kg + 1; k < limit; ++k) {
+        if (st.done[k]) break;
+        if (is_view_op(g->nodes[k])) continue;
+        if (g->nodes[k]->op == GGML_OP_SCALE && through_views(g->nodes[k]->src[0]) == gr && ggml_abi_op_param_f32(g->nodes[k], 1) == 0.0f) ks = k;
+        break;
+    }
+    if (ks < 0) return 0;
+    const ggml_tensor * sc = g->nodes[ks];
+    if (!is_f32_contig(sc) || ranges_overlap(sc, a) || ranges_overlap(sc, sm) || ranges_overlap(sc, as)) return 0;
+    // the score tensor has two readers in this pattern (the sort and the row pick); the permutation one (the view)
+    for (int j = i + 1; j < ks; ++j) {
+        const ggml_tensor * u = g->nodes[j];
+        if (j == kg || j == ka) continue;
+        if (!is_view_op(u) && ranges_overlap(sc, u)) return 0;
+        for (int sidx = 0; sidx < GGML_MAX_SRC; ++sidx)
+            if (u->src[sidx] && u->src[sidx] != gr && ranges_overlap(sc, u->src[sidx])) return 0;
+    }
+    const int groups = as->op_params[1] > 1 ? as->op_params[1] : 1, keep = as->op_params[1] > 1 ? as->op_params[2] : 1;
+    launch_router_softmax_topk(st.c->stream, TD(a), TD(sm), TD(as), TD(sc), (int) gr->src[1]->ne[0], groups, keep, ggml_abi_op_param_f32(sc, 0));
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 3;
+    mark_done(st, ka);
+    mark_done(st, kg);
+    mark_done(st, ks);
+    return 1;
+}
+
+// ADD(x, y) -> RMS_NORM(.) -> MUL(., w row): a residual update and the norm of the sublayer that follows in one launch (pre-norm models whose norms are RMS norms).
+// The sum stays a tensor of its own: the stream goes on from it.  Returns the nodes consumed at position i (0: no match)
+static int try_fuse_add_rms_norm(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * ad = g->nodes[i];
+    const ggml_tensor * x = ad->src[0], * y = ad->src[1];
+    if (!is_f32_contig(ad) || !is_f32_contig(x) || !is_f32_contig(y) || !same_shape(ad, x) || !same_shape(ad, y) || (ad->flags & GGML_TENSOR_FLAG_OUTPUT)) return 0;
+    int k1 = i + 1;
+    while (k1 < g->n_nodes && !st.done[k1] && is_view_op(g->nodes[k1])) ++k1;
+    if (k1 + 1 >= g->n_nodes || st.done[k1] || st.done[k1 + 1]) return 0;
+    const ggml_tensor * rn = g->nodes[k1], * ml = g->nodes[k1 + 1];
+    if (rn->op != GGML_OP_RMS_NORM || rn->src[0] != ad || ml->op != GGML_OP_MUL || !single_use(st, rn) || !is_f32_contig(ml) || !same_shape(ml, ad)) return 0;
+    const ggml_tensor * w = ml->src[0] == rn ? ml->src[1] : (ml->src[1] == rn ? ml->src[0] : nullptr);
+    if (!w || !is_row_of(w, ad)) return 0;
+    for (int j = k1 + 2; j < g->n_nodes; ++j)  // (a norm read by quantised products has forms of its own: quantised on the way, deferred into the product, assembled from split-K parts)
+        for (int sidx = 0; sidx < GGML_MAX_SRC; ++sidx)
+            if (g->nodes[j]->src[sidx] == ml && g->nodes[j]->op == GGML_OP_MUL_MAT && g->nodes[j]->src[0] && is_quant(g->nodes[j]->src[0]->type)) return 0;
+    if (st.sk_dst == x || st.sk_dst == y) return 0;
+    if (ranges_overlap(ml, ad) || ranges_overlap(ml, x) || ranges_overlap(ml, y) || ranges_overlap(ml, w) || ranges_overlap(ad, w)) return 0;
+    if ((ranges_overlap(ad, x) && ad->data != x->data) || (ranges_overlap(ad, y) && ad->data != y->data)) return 0;
+    launch_add_rms_norm_mul(st.c->stream, (const float *) x->data, (const float *) y->data, (float *) ad->data, (float *) ml->data, (const float *) w->data, ad->ne[0],
+                            ggml_abi_nrows(ad), ggml_abi_op_param_f32(rn, 0));
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 2;
+    mark_done(st, k1);
+    mark_done(st, k1 + 1);
+    return 1;
+}
+
+// RMS_NORM(o [DV, H, T]) -> MUL(., w) -> [RESHAPE] ... UNARY(gate; SiLU or sigmoid) -> MUL(., act): the norm, weight and gate behind a recurrence in one launch
+static int try_fuse_head_norm_gate(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * rn = g->nodes[i];
+    const ggml_tensor * o = rn->src[0];
+    if (o->type != GGML_TYPE_F32 || o->nb[0] != 4 || o->ne[3] != 1 || !is_f32_contig(rn) || !single_use(st, rn)) return 0;
+    // the three nodes behind the norm, views between them skipped: MUL by the weight, the gate's activation, MUL by it
+    int at[3] = {-1, -1, -1}, found = 0;
+    for (int k = i + 1; k < std::min(g->n_nodes, i + 10) && found < 3; ++k) {
+        if (st.done[k]) return 0;
+        if (is_view_op(g->nodes[k])) continue;
+        at[found++] = k;
+    }
+    if (found < 3) return 0;
+    const ggml_tensor * ml = g->nodes[at[0]], * un = g->nodes[at[1]], * out = g->nodes[at[2]];
+    if (ml->op != GGML_OP_MUL || ml->src[0] != rn || !single_use(st, ml) || !same_shape(ml, rn) || un->op != GGML_OP_UNARY || out->op != GGML_OP_MUL) return 0;
+    const ggml_tensor * w = ml->src[1];
+    const bool w_row = ggml_abi_nelements(w) == o->ne[0] && w->ne[0] == o->ne[0];
+    const bool w_heads = w->ne[0] == o->ne[0] && w->ne[1] == o->ne[1] && ggml_abi_nelements(w) == o->ne[0] * o->ne[1];
+    if (!is_f32_contig(w) || !(w_row || w_heads)) return 0;
+    const int uop = un->op_params[0];
+    if ((uop != GGML_UNARY_OP_SILU && uop != GGML_UNARY_OP_SIGMOID) || !single_use(st, un) || through_views(out->src[0]) != ml || out->src[1] != un) return 0;
+    const ggml_tensor * gate = un->src[0];
+    if (!is_f32_contig(gate) || !is_f32_contig(out) || ggml_abi_nelements(gate) != ggml_abi_nelements(o) || ggml_abi_nelements(out) != ggml_abi_nelements(o)) return 0;
+    // (the graph allocator runs these element-wise nodes in place: the result usually lies over o or over the gate — entry for entry, which the kernel allows: a wave
+    // reads its whole row for the sum of squares before it writes any of it, and the gate entry it reads is the one it replaces)
+    if ((ranges_overlap(out, o) && !(out->data == o->data && ggml_abi_is_contiguous(o))) || ranges_overlap(out, w) || (ranges_overlap(out, gate) && out->data != gate->data)) return 0;
+    launch_head_norm_gate(st.c->stream, TD(o), (const float *) w->data, w_row ? 0 : 1, (const float *) gate->data, uop == GGML_UNARY_OP_SIGMOID ? 1 : 0, (float *) out->data,
+                          ggml_abi_op_param_f32(rn, 0));
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 3;
+    for (int k = 0; k < 3; ++k) mark_done(st, at[k]);
+    return 1;
+}
+
 static int run_node(exec_state & st, int i);
 static bool try_fuse_geglu_bias(exec_state & st, int i) {
     ggml_cgraph * g = st.g;
@@ -1984,6 +2140,7 @@ static int run_node(exec_state & st, int i) {
             return 1;
 
         case GGML_OP_RMS_NORM: {
+            if (fuse) { const int r = try_fuse_head_norm_gate(st, i); if (r) return r; }
             // RMS_NORM -> MUL(norm, w): one kernel writing the MUL's output
             ggml_tensor * m = next(1);
             if (fuse && m && m->op == GGML_OP_MUL && single_use(st, n) && m->type == GGML_TYPE_F32 && m->nb[0] == 4) {
@@ -2170,6 +2327,10 @@ static int run_node(exec_state & st, int i) {
         }
 
         case GGML_OP_ADD: case GGML_OP_SUB: case GGML_OP_MUL: case GGML_OP_DIV: {
+            if (fuse && n->op == GGML_OP_ADD) {
+                const int used = try_fuse_add_rms_norm(st, i);
+                if (used) return used;
+            }
             if (fuse && n->op == GGML_OP_MUL) {
                 const int used = try_fuse_expert_sum(st, i);
                 if (used > 0) return used;
@@ -2304,7 +2465,45 @@ static int run_node(exec_state & st, int i) {
                     }
                 }
             }
-            launch_argsort(s, TD(a), TD(n), n->op_params[0] == 1 ? 1 : 0);
+            if (n->op_params[1] > 1) launch_argsort_grouped(s, TD(a), TD(n), n->op_params[1], n->op_params[2]);
+            else launch_argsort(s, TD(a), TD(n), n->op_params[0] == 1 ? 1 : 0);
+            c->st.kernel_launches++;
+            return 1;
+        }
+        case GGML_OP_SSM_CONV: {
+            const int taps = n->op_params[0];
+            if (n->op_params[2] == 1) {
+                timed_scope ts(c, "seq_conv", (double) ggml_abi_nbytes(n));
+                launch_seq_conv_store(s, TD(a), (float *) n->data, (const int32_t *) n->src[1]->data, (int) n->src[1]->ne[0], (const int32_t *) n->src[2]->data, (int) n->src[2]->ne[1], taps);
+            } else {
+                timed_scope ts(c, "seq_conv", (double) ggml_abi_nbytes(a) + (double) ggml_abi_nbytes(n));
+                launch_seq_conv(s, TD(a), (const float *) n->src[1]->data, n->src[2] ? (const float *) n->src[2]->data : nullptr, n->src[3] ? (const int32_t *) n->src[3]->data : nullptr,
+                                n->src[3] ? (int) n->src[3]->ne[0] : 0, TD(n), taps, n->op_params[1]);
+            }
+            c->st.kernel_launches++;
+            return 1;
+        }
+        case GGML_OP_RWKV_WKV6: case GGML_OP_GATED_LINEAR_ATTN: {
+            const bool wkv = n->op == GGML_OP_RWKV_WKV6;
+            const int kind = wkv ? SEQ_WKV6 : n->op_params[0];
+            const ggml_tensor * state = n->src[wkv ? 6 : 5], * tok = n->src[wkv ? 7 : 6], * info = n->src[wkv ? 8 : 7];
+            seq_rec_args ra;
+            ra.q = TD(n->src[0]); ra.k = TD(n->src[1]); ra.v = TD(n->src[2]); ra.g = TD(n->src[3]);
+            ra.p0 = (const float *) n->src[4]->data;
+            ra.p1 = wkv ? (const float *) n->src[5]->data : nullptr;
+            ra.state = (float *) state->data;
+            ra.state_stride = (int64_t) (state->nb[1] / 4);
+            ra.tok = (const int32_t *) tok->data;
+            ra.info = (const int32_t *) info->data;
+            ra.dst = TD(n);
+            ra.H = wkv ? n->op_params[0] : n->op_params[1];
+            ra.G = wkv ? ra.H : n->op_params[2];
+            ra.DK = (int) (n->src[0]->ne[0] / ra.G);
+            ra.DV = (int) (n->src[2]->ne[0] / ra.H);
+            ra.cap = wkv ? 0.0f : ggml_abi_op_param_f32(n, 4);
+            ra.qscale = wkv ? 1.0f : ggml_abi_op_param_f32(n, 5);
+            timed_scope ts(c, "seq_recurrence", (double) info->ne[1] * (double) state->nb[1] * 2.0);
+            launch_seq_recurrence(s, kind, ra, (int) info->ne[1]);
             c->st.kernel_launches++;
             return 1;
         }
@@ -2512,6 +2711,7 @@ static int run_node(exec_state & st, int i) {
         }
         case GGML_OP_SOFT_MAX: {
             const tdesc md = b ? TD(b) : TD(a);
+            if (fuse) { const int r = try_fuse_router_scores(st, i); if (r) return r; }
             // a decode step on the non-flash path: the probabilities have one reader, MUL_MAT(V^T view, p) — made inside that product
             if (fuse && c->opt.softmax_mm && n->ne[1] == 1 && !n->src[2] && ggml_abi_op_param_f32(n, 1) == 0.0f && a->type == GGML_TYPE_F32 && ggml_abi_is_contiguous(a) &&
                 single_use(st, n)) {
@@ -2624,7 +2824,8 @@ static int run_node(exec_state & st, int i) {
             if (fa_route(n) == 4) {
                 const tdesc md4 = m ? TD(m) : qd;
                 timed_scope ts(c, "attn_f32", (double) ggml_abi_nbytes(k) + (double) ggml_abi_nbytes(v));
-                launch_attn_f32(s, qd, kd, vd, m ? &md4 : nullptr, n->src[4] ? (const float *) n->src[4]->data : nullptr, n->src[5] ? (const float *) n->src[5]->data : nullptr, TD(n), p.scale);
+                launch_attn_f32(s, qd, kd, vd, m ? &md4 : nullptr, n->src[4] ? (const float *) n->src[4]->data : nullptr, n->src[5] ? (const float *) n->src[5]->data : nullptr, TD(n), p.scale,
+                                n->src[6] ? (const float *) n->src[6]->data : nullptr, p.logit_softcap);
                 c->st.kernel_launches++;
                 c->st.attn_f32_nodes++;
                 return 1;

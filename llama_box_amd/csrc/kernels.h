@@ -172,7 +172,9 @@ bool launch_mul_mat_id(hipStream_t s, const tdesc & as, const tdesc & b, const t
 bool attn_f32_applies(const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const tdesc & dst);
 // r12 (optional: r1 of every head, then r2 of every head): the mask then holds the DISTANCE between query and cell for visible pairs (-inf for hidden ones) and the score is
 // q.k * scale - r1 ln(1 + r2 distance)
-void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const float * r12, const tdesc & dst, float scale);
+// sig: per head a factor on the score, then per head a bias ([heads, 2]) — the weights are then sigmoid(score + bias), not a soft-max; softcap > 0: score <- cap tanh(score / cap)
+void launch_attn_f32(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc * mask, const float * sinks, const float * r12, const tdesc & dst, float scale,
+                     const float * sig = nullptr, float softcap = 0.0f);
 // ---- non-flash attention chain of a small batch over position lists (attn_nf.hip)
 size_t attn_nf_list_scratch_bytes(const tdesc & q, const tdesc & k, int * dq_out);
 bool launch_attn_nf_list(hipStream_t s, const tdesc & q, const tdesc & k, const tdesc & v, const tdesc & mask, const tdesc & dst, const int * lists, int list_stride,
@@ -377,6 +379,35 @@ void launch_repack_planes(hipStream_t s, int type, const void * src, void * dst,
 bool repack_q80_supported(int type, int64_t K, int64_t N, int64_t nb1);  // Q8_0: the panel copy of the 9 .. 32-column matrix-core kernel (repack.hip)
 void launch_repack_q80_panels(hipStream_t s, const void * src, void * dst, int64_t K, int64_t N, int64_t nb1);
 
+// ---- layers with state per sequence (seq.hip): short convolutions over a sequence's history and three recurrences over a matrix state per head
+void launch_seq_conv(hipStream_t s, const tdesc & x, const float * w, const float * state, const int32_t * hist, int hs, const tdesc & dst, int taps, int act);
+void launch_seq_conv_store(hipStream_t s, const tdesc & x, float * state, const int32_t * upd, int hs, const int32_t * info, int n_seqs, int taps);
+struct seq_rec_args {
+    tdesc q, k, v;             // [rows, T] f32 (rows contiguous): q / r, k and v of all heads
+    tdesc g;                   // wkv6: w_pre [D H, T]; delta: (b_pre, a_pre) [2 H, T]; mlstm: (i_pre, f_pre) [2 H, T]
+    const float * p0;          // wkv6: w0 [D H]; delta: A_log [H] then dt_bias [H]; mlstm: bias of (i, f) [2 H]
+    const float * p1;          // wkv6: u [D H]
+    float * state;             // per slot: H matrices of 4 ceil(DK / 4) DV values, then (mlstm) H x DK normaliser entries and H running maxima
+    int64_t state_stride;      // floats per slot
+    const int32_t * tok;
+    const int32_t * info;
+    tdesc dst;                 // [DV, H, T]
+    int DK, DV, H, G;          // G: key heads (head h reads q / k head h / (H / G))
+    float cap, qscale;
+};
+
+enum { SEQ_WKV6 = 0, SEQ_DELTA = 1, SEQ_MLSTM = 2 };
+int64_t seq_recurrence_state_floats(int kind, int H, int DK, int DV);
+bool seq_recurrence_ok(int DK, int DV);
+void launch_seq_recurrence(hipStream_t s, int kind, const seq_rec_args & a, int n_seqs);
+// SOFT_MAX over a router's logits, the (group-limited) descending ARGSORT of the scores, GET_ROWS of the k first and SCALE in one launch (n <= 256 experts)
+void launch_router_softmax_topk(hipStream_t s, const tdesc & logits, const tdesc & probs, const tdesc & ids, const tdesc & wts /* [1, k, T] */, int k, int groups, int keep, float wscale);
+// RMS_NORM per head -> MUL(weight: [DV] or [DV, H]) -> MUL(act(gate)), act SiLU (0) or sigmoid (1): o [DV, H, T] (rows contiguous), gate and d [DV H, T] contiguous
+void launch_head_norm_gate(hipStream_t s, const tdesc & o, const float * w, int w_per_head, const float * gate, int sigmoid_act, float * d, float eps);
+// ADD(x, y) -> RMS_NORM -> MUL(w): sum (may lie over x or y) and the normed rows d, all [n, rows] contiguous f32
+void launch_add_rms_norm_mul(hipStream_t s, const float * x, const float * y, float * sum, float * d, const float * w, int64_t n, int64_t rows, float eps);
+void launch_argsort_grouped(hipStream_t s, const tdesc & src, const tdesc & dst, int groups, int keep);  // descending; entries outside the `keep` groups with the largest maxima sort last
+
 // ---- code-object preload (round 4).  The HIP runtime loads a translation unit's device code on the FIRST launch of one of its kernels
 // (0.3 - 2 ms each, measured as idle gaps in front of the first prompt's kernels: 5.5 ms of a 64 ms prefill).  Every kernel file ends with
 // MI_TU_TOUCH(name): an empty kernel + a launcher; init_backend launches them all once per device, so the cost moves to start-up.
@@ -399,6 +430,7 @@ void tu_touch_fattn_mma(hipStream_t s);
 void tu_touch_tp_p2p(hipStream_t s);
 void tu_touch_kv_types(hipStream_t s);
 void tu_touch_repack(hipStream_t s);
+void tu_touch_seq(hipStream_t s);
 inline void preload_kernel_files(hipStream_t s) {
     tu_touch_kv_types(s);
     tu_touch_repack(s);
@@ -416,6 +448,7 @@ inline void preload_kernel_files(hipStream_t s) {
     tu_touch_attn_f32(s);
     tu_touch_fattn_mma(s);
     tu_touch_tp_p2p(s);
+    tu_touch_seq(s);
 }
 
 }  // namespace mi355x

@@ -282,6 +282,118 @@ void launch_topk_softmax(hipStream_t s, const tdesc & logits, const tdesc & ids,
     hipLaunchKernelGGL(k_topk_softmax, dim3((unsigned) logits.ne[1]), dim3(256), 0, s, logits, ids, wts, k);
 }
 
+// ------------------------------------------------------------------------------------------------ router: soft-max over all experts, group-limited top-k, scaled weights
+// one workgroup per token, a thread per expert (n <= 256): SOFT_MAX (k_soft_max_reg's arithmetic: block maximum, exponentials, their sum in double through the
+// same block tree, times the rounded reciprocal), the group-limited descending ARGSORT of the scores, GET_ROWS of the k first and SCALE — the nodes' own results
+__global__ void __launch_bounds__(256) k_router_softmax_topk(const tdesc a, const tdesc probs, const tdesc ids, const tdesc wts, const int k, const int groups, const int keep,
+                                                             const float wscale) {
+    __shared__ double shd[4];
+    __shared__ float shf[4];
+    __shared__ float p[256], gmax[256];
+    __shared__ int gkeep[256];
+    const int64_t t = blockIdx.x;
+    const int n = (int) a.ne[0], per = n / groups, i = threadIdx.x;
+    const float x = i < n ? ((const float *) (a.data + t * a.nb[1]))[i] * 1.0f : -INFINITY;
+    const float mx = block_max_f(x, shf);
+    const float e = i < n ? expf(x - mx) : 0.0f;
+    double sum = block_sum_d(i < n ? (double) e : 0.0, shd);
+    if (isnan(sum) || sum == 0.0) sum = -INFINITY;
+    const float inv = (float) (1.0 / sum);
+    const float pr = e * inv;
+    if (i < n) {
+        p[i] = pr;
+        ((float *) (probs.data + t * probs.nb[1]))[i] = pr;
+    }
+    __syncthreads();
+    if (i < groups) {
+        float m = p[i * per];
+        for (int q = 1; q < per; ++q) m = fmaxf(m, p[i * per + q]);
+        gmax[i] = m;
+    }
+    __syncthreads();
+    if (i < groups) {
+        int before = 0;
+        for (int o = 0; o < groups; ++o) before += (gmax[o] > gmax[i] || (gmax[o] == gmax[i] && o < i)) ? 1 : 0;
+        gkeep[i] = before < keep ? 1 : 0;
+    }
+    __syncthreads();
+    if (i < n) {
+        const float v = gkeep[i / per] ? pr : -INFINITY;
+        int before = 0;
+        for (int j = 0; j < n; ++j) {
+            const float u = gkeep[j / per] ? p[j] : -INFINITY;
+            before += (u > v || (u == v && j < i)) ? 1 : 0;
+        }
+        ((int32_t *) (ids.data + t * ids.nb[1]))[before] = i;
+        if (before < k) *(float *) (wts.data + (int64_t) before * wts.nb[1] + t * wts.nb[2]) = pr * wscale;
+    }
+}
+void launch_router_softmax_topk(hipStream_t s, const tdesc & logits, const tdesc & probs, const tdesc & ids, const tdesc & wts, int k, int groups, int keep, float wscale) {
+    if (logits.ne[1] == 0) return;
+    hipLaunchKernelGGL(k_router_softmax_topk, dim3((unsigned) logits.ne[1]), dim3(256), 0, s, logits, probs, ids, wts, k, groups, keep, wscale);
+}
+
+// ------------------------------------------------------------------------------------------------ residual sum and the RMS norm of the next sublayer
+// ADD(x, y) -> RMS_NORM -> MUL(., w): the stream's update and the norm that reads it in one launch; both results are written (the sum goes on as the residual).  The sum of
+// squares is f64 as in k_rms_norm.  A thread re-reads only entries of the sum it wrote itself, so the sum may lie over x or y.
+__global__ void __launch_bounds__(256) k_add_rms_norm_mul(const float * x, const float * y, float * sum, float * __restrict__ d, const float * __restrict__ w, const int64_t n, const float eps) {
+    __shared__ double sh[4];
+    const int64_t row = blockIdx.x;
+    const float * xr = x + row * n, * yr = y + row * n;
+    float * sr = sum + row * n;
+    double s = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = xr[i] + yr[i];
+        sr[i] = v;
+        s += (double) (v * v);
+    }
+    s = block_sum_d(s, sh);
+    const float mean = (float) (s / (double) n);
+    const float scale = 1.0f / sqrtf(mean + eps);
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = sr[i] * scale;
+        v = v * w[i];
+        d[row * n + i] = v;
+    }
+}
+void launch_add_rms_norm_mul(hipStream_t s, const float * x, const float * y, float * sum, float * d, const float * w, int64_t n, int64_t rows, float eps) {
+    if (rows == 0 || n == 0) return;
+    hipLaunchKernelGGL(k_add_rms_norm_mul, dim3((unsigned) rows), dim3(256), 0, s, x, y, sum, d, w, n, eps);
+}
+
+// ------------------------------------------------------------------------------------------------ per-head norm, weight and gate behind a recurrence
+// RMS_NORM over a head's entries, MUL by a weight (one row for all heads, or one entry per (head, entry)), MUL by act(gate): a wave per (head, token) row.
+// The sum of squares is f64 as in k_rms_norm, so the scale is the same f32 number.
+__global__ void __launch_bounds__(256) k_head_norm_gate(const tdesc o, const float * __restrict__ w, const int w_per_head, const float * gate, const int sigmoid_act,
+                                                        float * d, const float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t) blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t DV = o.ne[0], H = o.ne[1], rows = H * o.ne[2];
+    if (row >= rows) return;
+    const int64_t h = row % H, t = row / H;
+    const float * x = (const float *) (o.data + h * o.nb[1] + t * o.nb[2]);
+    double s = 0.0;
+    for (int64_t i = lane; i < DV; i += 64) s += (double) (x[i] * x[i]);
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    const float mean = (float) (s / (double) DV);
+    const float scale = 1.0f / sqrtf(mean + eps);
+    const float * __restrict__ wr = w + (w_per_head ? h * DV : 0);
+    const float * gr = gate + (t * H + h) * DV;
+    float * y = d + (t * H + h) * DV;
+    for (int64_t i = lane; i < DV; i += 64) {
+        float v = x[i] * scale;
+        v = v * wr[i];
+        const float g = gr[i];
+        const float a = sigmoid_act ? 1.f / (1.f + expf(-g)) : silu_f(g);
+        y[i] = v * a;
+    }
+}
+void launch_head_norm_gate(hipStream_t s, const tdesc & o, const float * w, int w_per_head, const float * gate, int sigmoid_act, float * d, float eps) {
+    const int64_t rows = o.ne[1] * o.ne[2];
+    if (rows == 0 || o.ne[0] == 0) return;
+    hipLaunchKernelGGL(k_head_norm_gate, dim3((unsigned) ((rows + 3) / 4)), dim3(256), 0, s, o, w, w_per_head, gate, sigmoid_act, d, eps);
+}
+
 // ------------------------------------------------------------------------------------------------ ARGSORT
 // one workgroup per row: element i's place is the number of elements that sort before it (ties keep their index order), so the result is the
 // stable sort's permutation; rows of up to a few thousand entries (router logits)
@@ -306,6 +418,44 @@ void launch_argsort(hipStream_t s, const tdesc & src, const tdesc & dst, int des
     const int64_t rows = src.ne[1] * src.ne[2] * src.ne[3];
     if (rows == 0) return;
     hipLaunchKernelGGL(k_argsort, dim3((unsigned) rows), dim3(256), 0, s, src, dst, descending);
+}
+
+// the same (descending) for a router whose experts form `groups` equal groups of neighbours: only entries of the `keep` groups with the largest maxima may
+// come first — the others are ranked as if they were -inf (ties by index), so the leading columns hold the largest entries of the kept groups
+__global__ void __launch_bounds__(256) k_argsort_grouped(const tdesc a, const tdesc d, const int groups, const int keep) {
+    __shared__ float gmax[256];
+    __shared__ int gkeep[256];
+    const int64_t row = blockIdx.x;
+    const int64_t i1 = row % a.ne[1], i2 = (row / a.ne[1]) % a.ne[2], i3 = row / (a.ne[1] * a.ne[2]);
+    const float * __restrict__ x = (const float *) (a.data + i1 * a.nb[1] + i2 * a.nb[2] + i3 * a.nb[3]);
+    int32_t * __restrict__ y = (int32_t *) (d.data + i1 * d.nb[1] + i2 * d.nb[2] + i3 * d.nb[3]);
+    const int n = (int) a.ne[0], per = n / groups;
+    for (int g = threadIdx.x; g < groups; g += blockDim.x) {
+        float m = x[g * per];
+        for (int e = 1; e < per; ++e) m = fmaxf(m, x[g * per + e]);
+        gmax[g] = m;
+    }
+    __syncthreads();
+    for (int g = threadIdx.x; g < groups; g += blockDim.x) {
+        int before = 0;
+        for (int o = 0; o < groups; ++o) before += (gmax[o] > gmax[g] || (gmax[o] == gmax[g] && o < g)) ? 1 : 0;
+        gkeep[g] = before < keep ? 1 : 0;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = gkeep[i / per] ? x[i] : -INFINITY;
+        int before = 0;
+        for (int j = 0; j < n; ++j) {
+            const float u = gkeep[j / per] ? x[j] : -INFINITY;
+            before += (u > v || (u == v && j < i)) ? 1 : 0;
+        }
+        y[before] = i;
+    }
+}
+void launch_argsort_grouped(hipStream_t s, const tdesc & src, const tdesc & dst, int groups, int keep) {
+    const int64_t rows = src.ne[1] * src.ne[2] * src.ne[3];
+    if (rows == 0) return;
+    hipLaunchKernelGGL(k_argsort_grouped, dim3((unsigned) rows), dim3(256), 0, s, src, dst, groups, keep);
 }
 
 // ------------------------------------------------------------------------------------------------ small fused element-wise forms

@@ -1,0 +1,338 @@
+// seq.hip — layers that carry STATE from token to token of a sequence, over a batch that mixes sequences freely (prompt portions of some beside
+// single tokens of others).  The scheduler describes the batch with four small integer inputs:
+//   hist [hs, T]      for token t and d = 1 .. hs: where the d-th token BEFORE t of the same sequence is found — a row of this batch (>= 0), nowhere (-1: before
+//                     the sequence's start, reads as zero), or the sequence's state (-2 - (slot * 64 + age): the age-th most recent token before this batch);
+//   upd  [hs, n_seq]  the same codes for the state AFTER the batch: entry a of sequence s is where its new age-a token comes from;
+//   tok  [T]          the batch rows grouped by sequence, each group in position order;
+//   info [4, n_seq]   per sequence of the batch: (first entry of its group in tok, number of entries, state slot, 1 when the sequence starts in this batch).
+// A sequence that starts reads no state at all (zeros), so a slot taken over by a new request needs no clearing.
+//
+// Kernels:
+//   k_seq_conv        short causal convolution per channel over a sequence's history (taps inputs, the last one the token's own), optionally followed by SiLU;
+//                     several weight sets over the same input give several outputs (a token shift h + (h_prev - h) mu is the 2-tap case with weights (mu, 1 - mu))
+//   k_seq_conv_store  the last taps - 1 inputs of every sequence of the batch become its state
+//   k_seq_wkv6        o_t = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T, w = exp(-exp(w_pre + w0)) per key channel
+//   k_seq_delta       gated delta rule: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q — unit-length q, k, sigmoid beta and the decay
+//                     g = exp(-exp(A_log) softplus(a + dt_bias)) computed here from the raw projections
+//   k_seq_mlstm       matrix memory with exponential gates under a running maximum m: m' = max(f + m, i); S <- e^(f + m - m') S + e^(i - m') k v^T; n likewise with k;
+//                     o = S^T q / (max(|n . q|, e^(-m')) + 1e-6); log gates capped by cap tanh(. / cap), f through log-sigmoid
+// All arithmetic is f32; the state is f32.  The three recurrences share one thread layout: a wave per (sequence of the batch, head, 4 value columns); value column j
+// of the head's state matrix is held by SIXTEEN neighbouring lanes (a DPP row), each owning a sixteenth of the key rows (neighbours) in registers; dot products over the key
+// rows are partial sums per lane joined across the sixteen by four DPP permutations (every lane then holds the same sum).  The vectors of several tokens are staged in
+// LDS a block ahead.  In memory a head's matrix is kept in the order the lanes read it ([register][column][ks]: one coalesced load per register).
+#include <algorithm>
+#include <cstdlib>
+
+#include "dev_util.h"
+#include "kernels.h"
+
+namespace mi355x {
+
+constexpr int SEQ_MAX_TAPS = 16;
+constexpr int SEQ_MAX_DK = 256;  // key rows of a head (16 lanes x up to 16 rows each)
+
+__device__ __forceinline__ float seq_hist_value(const int code, const int c, const int64_t C, const int taps, const char * __restrict__ xdata, const int64_t x_nb1,
+                                                const float * __restrict__ state) {
+    if (code >= 0) return ((const float *) (xdata + (int64_t) code * x_nb1))[c];
+    if (code == -1) return 0.0f;
+    const int cd = -2 - code, slot = cd >> 6, age = cd & 63;
+    return state[((int64_t) slot * (taps - 1) + age) * C + c];
+}
+
+__device__ __forceinline__ float seq_silu(const float z) { return z / (1.0f + expf(-z)); }
+
+// y[c, t, m] = act(sum_j w[j, c, m] * x_(t - (taps - 1 - j))[c])
+__global__ void __launch_bounds__(256) k_seq_conv(const tdesc x, const float * __restrict__ w, const float * __restrict__ state, const int32_t * __restrict__ hist, const int hs,
+                                                  const tdesc dst, const int taps, const int act) {
+    const int64_t C = x.ne[0], t = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    float xv[SEQ_MAX_TAPS];  // xv[d]: the input d tokens back
+    xv[0] = ((const float *) (x.data + t * x.nb[1]))[c];
+#pragma unroll
+    for (int d = 1; d < SEQ_MAX_TAPS; ++d) xv[d] = d < taps ? seq_hist_value(hist[t * hs + d - 1], c, C, taps, x.data, x.nb[1], state) : 0.0f;
+    for (int64_t m = 0; m < dst.ne[2]; ++m) {
+        const float * __restrict__ wc = w + (m * C + c) * taps;
+        float y = 0.0f;
+#pragma unroll
+        for (int d = SEQ_MAX_TAPS - 1; d >= 0; --d)
+            if (d < taps) y = fmaf(wc[taps - 1 - d], xv[d], y);  // oldest input first
+        ((float *) (dst.data + t * dst.nb[1] + m * dst.nb[2]))[c] = act ? seq_silu(y) : y;
+    }
+}
+
+__global__ void __launch_bounds__(256) k_seq_conv_store(const tdesc x, float * __restrict__ state, const int32_t * __restrict__ upd, const int hs, const int32_t * __restrict__ info,
+                                                        const int taps) {
+    const int64_t C = x.ne[0], s = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int slot = info[4 * s + 2];
+    float nv[SEQ_MAX_TAPS - 1];
+#pragma unroll
+    for (int a = 0; a < SEQ_MAX_TAPS - 1; ++a) nv[a] = a < taps - 1 ? seq_hist_value(upd[s * hs + a], c, C, taps, x.data, x.nb[1], state) : 0.0f;
+#pragma unroll
+    for (int a = 0; a < SEQ_MAX_TAPS - 1; ++a)
+        if (a < taps - 1) state[((int64_t) slot * (taps - 1) + a) * C + c] = nv[a];  // (every value was read before the first is written: the rows shift in place)
+}
+
+void launch_seq_conv(hipStream_t s, const tdesc & x, const float * w, const float * state, const int32_t * hist, int hs, const tdesc & dst, int taps, int act) {
+    if (x.ne[1] == 0 || x.ne[0] == 0) return;
+    hipLaunchKernelGGL(k_seq_conv, dim3((unsigned) ((x.ne[0] + 255) / 256), (unsigned) x.ne[1]), dim3(256), 0, s, x, w, state, hist, hs, dst, taps, act);
+}
+void launch_seq_conv_store(hipStream_t s, const tdesc & x, float * state, const int32_t * upd, int hs, const int32_t * info, int n_seqs, int taps) {
+    if (n_seqs == 0 || x.ne[0] == 0 || taps < 2) return;
+    hipLaunchKernelGGL(k_seq_conv_store, dim3((unsigned) ((x.ne[0] + 255) / 256), (unsigned) n_seqs), dim3(256), 0, s, x, state, upd, hs, info, taps);
+}
+
+// ------------------------------------------------------------------------------------------------ the recurrences
+__device__ __forceinline__ float quad_sum(float x) {  // sum over the 16 lanes of a row (the lanes of one value column); every lane gets the same bits
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xF, 0xF, true));   // quad lanes (1, 0, 3, 2)
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x4E, 0xF, 0xF, true));   // quad lanes (2, 3, 0, 1): the four hold their quad's sum
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x141, 0xF, 0xF, true));  // mirrored within each half row: the other quad of the half
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x140, 0xF, 0xF, true));  // mirrored within the row: the other half
+    return x;
+}
+__device__ __forceinline__ float seq_softplus(const float z) { return fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z))); }
+__device__ __forceinline__ float seq_log_sigmoid(const float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
+
+
+// One WAVE per (sequence of the batch, head, group of 4 value columns).  The tokens' vectors come in blocks of TB tokens: while block b is worked on out of LDS, block
+// b + 1 travels from memory into registers (one trip to memory per block, not per token) and is written to the other LDS buffer at the end; the batch rows of block b + 2
+// are fetched at the same time, so that no load ever waits for an address that is itself on its way.  A token's entries in a block: k [DK], q [DK], (wkv6: decay [DK]),
+// the wave's 4 values, (delta / matrix memory: the head's two raw gates).
+constexpr int SEQ_COLS = 4;        // value columns of a wave
+constexpr int SEQ_LPC = 16;        // lanes per value column: each owns a sixteenth of the key rows
+constexpr int SEQ_NV = 32;         // registers a lane lends to the block on its way
+constexpr int SEQ_MAX_TB = 16;     // tokens of a block at most
+
+// key rows a lane owns: a sixteenth of the head's rows, rounded up to whole groups of four (its rows are neighbours, read from LDS sixteen bytes at a time)
+static inline __host__ __device__ int seq_rows_per_lane(const int DK) { return (((DK + SEQ_LPC - 1) / SEQ_LPC) + 3) / 4 * 4; }
+
+template <int KIND, int R, bool EXACT>   // R: key rows per lane at most (a multiple of 4); EXACT: exactly R (no test around a group of four rows)
+__global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, const int TB) {
+    __shared__ __attribute__((aligned(16))) float blk[2][SEQ_NV * 64];
+    __shared__ int rows_of[2][SEQ_MAX_TB];
+    const int s = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * SEQ_COLS, lane = threadIdx.x;
+    const int begin = A.info[4 * s], count = A.info[4 * s + 1], slot = A.info[4 * s + 2], reset = A.info[4 * s + 3];
+    const int DK = A.DK, DV = A.DV, H = A.H;
+    const int j = j0 + (lane >> 4), ks = lane & (SEQ_LPC - 1);
+    const bool col = j < DV;
+    const int RL = seq_rows_per_lane(DK), KP = SEQ_LPC * RL;  // lane ks owns rows ks RL .. ks RL + RL - 1; a token's key-sized vectors are padded with zeros to KP entries
+    const int kh = KIND == SEQ_WKV6 ? h : h / (H / A.G);
+    const int off_w = 2 * KP, off_v = KIND == SEQ_WKV6 ? 3 * KP : 2 * KP, off_g = off_v + SEQ_COLS;
+    const int per_tok = max(64, off_g + (KIND == SEQ_WKV6 ? 0 : 4));  // (at least a wave's stride: the walk over a block's entries then crosses at most one token per step)
+    float * __restrict__ Sm = A.state + (int64_t) slot * A.state_stride + (int64_t) h * RL * DV * SEQ_LPC;
+    float * __restrict__ Nm = A.state + (int64_t) slot * A.state_stride + (int64_t) H * RL * DV * SEQ_LPC + (int64_t) h * DK;
+    float * __restrict__ Mm = A.state + (int64_t) slot * A.state_stride + (int64_t) H * RL * DV * SEQ_LPC + (int64_t) H * DK + h;
+    float S[R], nn[R], uu[R];
+#pragma unroll
+    for (int ii = 0; ii < R; ++ii) {
+        // (no branch around a load: an entry that does not exist reads entry 0 and is dropped — the loads of all registers are then in flight together)
+        const int i = ks * RL + ii;
+        const bool ok = ii < RL && i < DK;
+        const float sv = Sm[(ok && col) ? ((int64_t) ii * DV + j) * SEQ_LPC + ks : 0];
+        S[ii] = (ok && col && !reset) ? sv : 0.0f;
+        if (KIND == SEQ_MLSTM) { const float nv = Nm[ok ? i : 0]; nn[ii] = (ok && !reset) ? nv : 0.0f; } else nn[ii] = 0.0f;
+        if (KIND == SEQ_WKV6) { const float uv = A.p1[h * DK + (ok ? i : 0)]; uu[ii] = ok ? uv : 0.0f; } else uu[ii] = 0.0f;
+    }
+    float mrun = (KIND == SEQ_MLSTM && !reset) ? *Mm : 0.0f;
+    const float a_exp = KIND == SEQ_DELTA ? expf(A.p0[h]) : 0.0f;
+    const float dt_b = KIND == SEQ_DELTA ? A.p0[H + h] : 0.0f;
+    const float bi = KIND == SEQ_MLSTM ? A.p0[h] : 0.0f, bf = KIND == SEQ_MLSTM ? A.p0[H + h] : 0.0f;
+
+    // entry e = lane + 64 i of a block (token u = e / per_tok, field f = e % per_tok) read from memory; `rows`: the block's batch rows
+    auto fetch = [&](const int * rows, const int n_tok, float (&pre)[SEQ_NV]) {
+        int u = lane >= per_tok ? 1 : 0, f = lane >= per_tok ? lane - per_tok : lane;  // (no loop inside: the 32 steps are one run of straight code)
+#pragma unroll
+        for (int i = 0; i < SEQ_NV; ++i) {
+            // which tensor, which entry: selected without branches, an entry that does not exist reads entry 0 of the block's first token (32 loads in flight together)
+            const bool is_k = f < KP, is_q = !is_k && f < 2 * KP, is_w = KIND == SEQ_WKV6 && !is_k && !is_q && f < off_v, is_v = !is_k && !is_q && !is_w && f < off_g;
+            const int fe = is_k ? f : is_q ? f - KP : is_w ? f - off_w : is_v ? f - off_v : f - off_g;
+            const bool valid = u < n_tok && (is_v ? j0 + fe < DV : (is_k || is_q || is_w) ? fe < DK : (KIND != SEQ_WKV6 && fe < 2));
+            const char * base = is_k ? A.k.data : is_q ? A.q.data : is_v ? A.v.data : A.g.data;
+            const int64_t nb1 = is_k ? A.k.nb[1] : is_q ? A.q.nb[1] : is_v ? A.v.nb[1] : A.g.nb[1];
+            const int idx = (is_k || is_q) ? kh * DK + fe : is_w ? h * DK + fe : is_v ? h * DV + j0 + fe : fe * H + h;
+            const int64_t t = rows[valid ? u : 0];
+            float val = ((const float *) (base + t * nb1))[valid ? idx : 0];
+            if (KIND == SEQ_WKV6) {
+                const float off = A.p0[(is_w && valid) ? h * DK + fe : 0];
+                val = is_w ? val + off : val;
+            }
+            pre[i] = valid ? val : 0.0f;
+            f += 64;
+            const bool over = f >= per_tok;
+            f = over ? f - per_tok : f;
+            u = over ? u + 1 : u;
+        }
+    };
+    auto park = [&](float * dstb, const float (&pre)[SEQ_NV]) {
+        int f = lane >= per_tok ? lane - per_tok : lane;
+#pragma unroll
+        for (int i = 0; i < SEQ_NV; ++i) {
+            if (lane + 64 * i < TB * per_tok) dstb[lane + 64 * i] = (KIND == SEQ_WKV6 && f >= off_w && f < off_v) ? expf(-expf(pre[i])) : pre[i];
+            f += 64;
+            f = f >= per_tok ? f - per_tok : f;
+        }
+    };
+    float pre[SEQ_NV];
+    if (lane < SEQ_MAX_TB) {
+        rows_of[0][lane] = lane < count ? A.tok[begin + lane] : 0;
+        rows_of[1][lane] = TB + lane < count ? A.tok[begin + TB + lane] : 0;
+    }
+    __syncthreads();
+    fetch(rows_of[0], min(TB, count), pre);
+    park(blk[0], pre);
+    __syncthreads();
+    for (int b0 = 0, b = 0; b0 < count; b0 += TB, ++b) {
+        const int n_here = min(TB, count - b0), n_next = min(TB, count - b0 - TB);
+        const float * cur = blk[b & 1];
+        const int * trow = rows_of[b & 1];
+        int row_after = 0;
+        if (n_next > 0) {
+            fetch(rows_of[(b + 1) & 1], n_next, pre);
+            if (lane < TB && b0 + 2 * TB + lane < count) row_after = A.tok[begin + b0 + 2 * TB + lane];
+        }
+        for (int u = 0; u < n_here; ++u) {
+            const float * lt = cur + u * per_tok;
+            const float4 * k4 = (const float4 *) (lt + ks * RL), * q4 = (const float4 *) (lt + KP + ks * RL), * w4 = (const float4 *) (lt + off_w + ks * RL);
+            const float vj = lt[off_v + (lane >> 4)];
+            float o = 0.0f;
+            if (KIND == SEQ_WKV6) {
+                float p0 = 0.0f, p1 = 0.0f, p2 = 0.0f, p3 = 0.0f;
+#pragma unroll
+                for (int m = 0; m < R / 4; ++m) {
+                    if (EXACT || 4 * m < RL) {
+                        const float4 kk = k4[m], rq = q4[m], ww = w4[m];
+                        const float kv0 = kk.x * vj, kv1 = kk.y * vj, kv2 = kk.z * vj, kv3 = kk.w * vj;
+                        p0 = fmaf(fmaf(uu[4 * m], kv0, S[4 * m]), rq.x, p0);
+                        p1 = fmaf(fmaf(uu[4 * m + 1], kv1, S[4 * m + 1]), rq.y, p1);
+                        p2 = fmaf(fmaf(uu[4 * m + 2], kv2, S[4 * m + 2]), rq.z, p2);
+                        p3 = fmaf(fmaf(uu[4 * m + 3], kv3, S[4 * m + 3]), rq.w, p3);
+                        S[4 * m] = fmaf(ww.x, S[4 * m], kv0);
+                        S[4 * m + 1] = fmaf(ww.y, S[4 * m + 1], kv1);
+                        S[4 * m + 2] = fmaf(ww.z, S[4 * m + 2], kv2);
+                        S[4 * m + 3] = fmaf(ww.w, S[4 * m + 3], kv3);
+                    }
+                }
+                o = quad_sum((p0 + p1) + (p2 + p3));
+            } else if (KIND == SEQ_DELTA) {
+                const float b_pre = lt[off_g], a_pre = lt[off_g + 1];
+                const float beta = 1.0f / (1.0f + expf(-b_pre));
+                const float gdec = expf(-a_exp * seq_softplus(a_pre + dt_b));
+                float kn[R], qn[R];
+                float k2a = 0.0f, k2b = 0.0f, q2a = 0.0f, q2b = 0.0f;
+#pragma unroll
+                for (int m = 0; m < R / 4; ++m) {
+                    float4 kk = make_float4(0.f, 0.f, 0.f, 0.f), qq = kk;
+                    if (EXACT || 4 * m < RL) { kk = k4[m]; qq = q4[m]; }
+                    kn[4 * m] = kk.x; kn[4 * m + 1] = kk.y; kn[4 * m + 2] = kk.z; kn[4 * m + 3] = kk.w;
+                    qn[4 * m] = qq.x; qn[4 * m + 1] = qq.y; qn[4 * m + 2] = qq.z; qn[4 * m + 3] = qq.w;
+                    k2a = fmaf(kk.x, kk.x, fmaf(kk.z, kk.z, k2a));
+                    k2b = fmaf(kk.y, kk.y, fmaf(kk.w, kk.w, k2b));
+                    q2a = fmaf(qq.x, qq.x, fmaf(qq.z, qq.z, q2a));
+                    q2b = fmaf(qq.y, qq.y, fmaf(qq.w, qq.w, q2b));
+                }
+                const float kinv = 1.0f / sqrtf(quad_sum(k2a + k2b) + 1e-6f), qinv = 1.0f / sqrtf(quad_sum(q2a + q2b) + 1e-6f) * A.qscale;
+                float d0 = 0.0f, d1 = 0.0f, d2 = 0.0f, d3 = 0.0f;
+#pragma unroll
+                for (int m = 0; m < R / 4; ++m) {
+                    if (EXACT || 4 * m < RL) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { kn[4 * m + e] *= kinv; S[4 * m + e] *= gdec; }
+                        d0 = fmaf(S[4 * m], kn[4 * m], d0);
+                        d1 = fmaf(S[4 * m + 1], kn[4 * m + 1], d1);
+                        d2 = fmaf(S[4 * m + 2], kn[4 * m + 2], d2);
+                        d3 = fmaf(S[4 * m + 3], kn[4 * m + 3], d3);
+                    }
+                }
+                const float uw = beta * (vj - quad_sum((d0 + d1) + (d2 + d3)));
+                float p0 = 0.0f, p1 = 0.0f, p2 = 0.0f, p3 = 0.0f;
+#pragma unroll
+                for (int m = 0; m < R / 4; ++m) {
+                    if (EXACT || 4 * m < RL) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) S[4 * m + e] = fmaf(kn[4 * m + e], uw, S[4 * m + e]);
+                        p0 = fmaf(S[4 * m], qn[4 * m] * qinv, p0);
+                        p1 = fmaf(S[4 * m + 1], qn[4 * m + 1] * qinv, p1);
+                        p2 = fmaf(S[4 * m + 2], qn[4 * m + 2] * qinv, p2);
+                        p3 = fmaf(S[4 * m + 3], qn[4 * m + 3] * qinv, p3);
+                    }
+                }
+                o = quad_sum((p0 + p1) + (p2 + p3));
+            } else {
+                const float i_raw = lt[off_g] + bi, f_raw = lt[off_g + 1] + bf;
+                const float ig = A.cap * tanhf(i_raw / A.cap), fg = seq_log_sigmoid(A.cap * tanhf(f_raw / A.cap));
+                const float m_new = fmaxf(fg + mrun, ig);
+                const float ea = expf(fg + mrun - m_new), eb = expf(ig - m_new);
+                mrun = m_new;
+                float n0 = 0.0f, n1 = 0.0f, e0 = 0.0f, e1 = 0.0f;
+#pragma unroll
+                for (int m = 0; m < R / 4; ++m) {
+                    if (EXACT || 4 * m < RL) {
+                        const float4 kk = k4[m], qq = q4[m];
+                        const float kf[4] = {kk.x, kk.y, kk.z, kk.w}, qf[4] = {qq.x * A.qscale, qq.y * A.qscale, qq.z * A.qscale, qq.w * A.qscale};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            S[4 * m + e] = fmaf(eb * kf[e], vj, ea * S[4 * m + e]);
+                            nn[4 * m + e] = fmaf(eb, kf[e], ea * nn[4 * m + e]);
+                        }
+                        n0 = fmaf(S[4 * m], qf[0], fmaf(S[4 * m + 2], qf[2], n0));
+                        n1 = fmaf(S[4 * m + 1], qf[1], fmaf(S[4 * m + 3], qf[3], n1));
+                        e0 = fmaf(nn[4 * m], qf[0], fmaf(nn[4 * m + 2], qf[2], e0));
+                        e1 = fmaf(nn[4 * m + 1], qf[1], fmaf(nn[4 * m + 3], qf[3], e1));
+                    }
+                }
+                const float num = quad_sum(n0 + n1), den = quad_sum(e0 + e1);
+                o = num / (fmaxf(fabsf(den), expf(-m_new)) + 1e-6f);
+            }
+            if (col && ks == 0) ((float *) (A.dst.data + (int64_t) h * A.dst.nb[1] + (int64_t) trow[u] * A.dst.nb[2]))[j] = o;
+        }
+        __syncthreads();  // (every lane has finished with this block's batch rows before they are replaced)
+        if (n_next > 0) {
+            park(blk[(b + 1) & 1], pre);
+            if (lane < TB) rows_of[b & 1][lane] = row_after;
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int ii = 0; ii < R; ++ii) {
+        const int i = ks * RL + ii;
+        const bool ok = ii < RL && i < DK;
+        if (col && ok) Sm[((int64_t) ii * DV + j) * SEQ_LPC + ks] = S[ii];
+        if (KIND == SEQ_MLSTM && j0 == 0 && lane < SEQ_LPC && ok) Nm[i] = nn[ii];
+    }
+    if (KIND == SEQ_MLSTM && j0 == 0 && lane == 0) *Mm = mrun;
+}
+
+// floats of state one slot needs
+int64_t seq_recurrence_state_floats(int kind, int H, int DK, int DV) {
+    return (int64_t) H * seq_rows_per_lane(DK) * DV * SEQ_LPC + (kind == SEQ_MLSTM ? (int64_t) H * DK + H : 0);
+}
+// (a lane holds up to 64 key rows of its column; a token's entries must fit the registers a wave lends to a block)
+bool seq_recurrence_ok(int DK, int DV) { return DK >= 1 && DK <= SEQ_MAX_DK && DV >= 1 && 3 * SEQ_LPC * seq_rows_per_lane(DK) + SEQ_COLS + 4 <= SEQ_NV * 64; }
+
+template <int KIND>
+static void seq_recurrence_launch(hipStream_t s, const seq_rec_args & a, int n_seqs) {
+    const int RL = seq_rows_per_lane(a.DK);
+    const int per_tok = std::max(64, (KIND == SEQ_WKV6 ? 3 : 2) * SEQ_LPC * RL + SEQ_COLS + (KIND == SEQ_WKV6 ? 0 : 4));
+    int TB = std::max(1, std::min(SEQ_MAX_TB, SEQ_NV * 64 / per_tok));
+    static const int tb_env = getenv("GGML_MI355X_SEQ_TB") ? atoi(getenv("GGML_MI355X_SEQ_TB")) : 0;  // (lab switch: fewer tokens per block)
+    if (tb_env > 0) TB = std::min(TB, tb_env);
+    const dim3 grid((unsigned) n_seqs, (unsigned) a.H, (unsigned) ((a.DV + SEQ_COLS - 1) / SEQ_COLS));
+#define MI_SEQ_REC(RR) do { if (RL == RR) hipLaunchKernelGGL((k_seq_recurrence<KIND, RR, true>), grid, dim3(64), 0, s, a, TB); \
+                            else hipLaunchKernelGGL((k_seq_recurrence<KIND, RR, false>), grid, dim3(64), 0, s, a, TB); } while (0)
+    if (RL <= 4) MI_SEQ_REC(4);
+    else if (RL <= 8) MI_SEQ_REC(8);
+    else MI_SEQ_REC(16);
+#undef MI_SEQ_REC
+}
+void launch_seq_recurrence(hipStream_t s, int kind, const seq_rec_args & a, int n_seqs) {
+    if (n_seqs == 0 || a.H == 0) return;
+    if (kind == SEQ_WKV6) seq_recurrence_launch<SEQ_WKV6>(s, a, n_seqs);
+    else if (kind == SEQ_DELTA) seq_recurrence_launch<SEQ_DELTA>(s, a, n_seqs);
+    else seq_recurrence_launch<SEQ_MLSTM>(s, a, n_seqs);
+}
+
+MI_TU_TOUCH(seq)
+
+}  // namespace mi355x
