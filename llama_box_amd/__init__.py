@@ -167,6 +167,10 @@ _SIGS = {
     "llm_kv_clear": (None, [_P]), "llm_kv_seq_rm": (_I, [_P, _I, _I, _I]), "llm_kv_seq_add": (_I, [_P, _I, _I, _I, _I]), "llm_last_graph": (C.POINTER(CGraph), [_P]), "llm_context_cache_tensor": (TP, [_P, _I, _I]),
     "llm_sample_greedy": (C.c_int32, [_P, _I]), "llm_token_probabilities": (_I, [_P, _I, _I, C.POINTER(C.c_int32), C.POINTER(C.c_float)]),
     "llm_last_timings": (None, [_P, C.POINTER(C.c_double)]),
+    "ggml_flash_attn_ext_set_sigmoid": (None, [TP, TP]), "ggml_argsort_grouped": (TP, [_P, TP, _I, _I]),
+    "ggml_seq_conv": (TP, [_P, TP, TP, TP, TP, _I]), "ggml_seq_conv_store": (TP, [_P, TP, TP, TP, TP, _I]),
+    "ggml_seq_wkv6": (TP, [_P, TP, TP, TP, TP, TP, TP, TP, TP, TP, _I]), "ggml_seq_gated_delta": (TP, [_P, TP, TP, TP, TP, TP, TP, TP, TP, _I, _I]),
+    "ggml_seq_mlstm": (TP, [_P, TP, TP, TP, TP, TP, TP, TP, TP, _I, _F]), "ggml_seq_state_size": (C.c_int64, [_I, _I, _I, _I]),
 }
 
 _host = None

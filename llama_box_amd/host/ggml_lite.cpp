@@ -13,6 +13,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
 #include <map>
 #include <string>
@@ -579,6 +580,93 @@ void ggml_flash_attn_ext_add_log_distance(struct ggml_tensor * a, struct ggml_te
     LITE_ASSERT(a->op == GGML_OP_FLASH_ATTN_EXT && a->src[3] != nullptr && a->src[3]->type == GGML_TYPE_F32);
     LITE_ASSERT(r12->type == GGML_TYPE_F32 && r12->ne[0] == a->src[0]->ne[2] && r12->ne[1] == 2 && ggml_is_contiguous(r12));
     a->src[5] = r12;
+}
+void ggml_flash_attn_ext_set_sigmoid(struct ggml_tensor * a, struct ggml_tensor * fb) {
+    LITE_ASSERT(a->op == GGML_OP_FLASH_ATTN_EXT && a->src[3] != nullptr && a->src[3]->type == GGML_TYPE_F32 && a->src[4] == nullptr);
+    LITE_ASSERT(fb->type == GGML_TYPE_F32 && fb->ne[0] == a->src[0]->ne[2] && fb->ne[1] == 2 && ggml_is_contiguous(fb));
+    a->src[6] = fb;
+}
+struct ggml_tensor * ggml_argsort_grouped(struct ggml_context * ctx, struct ggml_tensor * a, int groups, int keep) {
+    LITE_ASSERT(groups >= 1 && keep >= 1 && keep <= groups && a->ne[0] % groups == 0);
+    ggml_tensor * r = ggml_argsort(ctx, a, 1);
+    r->op_params[1] = groups;
+    r->op_params[2] = keep;
+    return r;
+}
+
+// ---- ops over sequence state: this harness's own operand layouts, marked by op_params[3] (the backend refuses the op numbers without the mark)
+static const int32_t SEQ_OP_TAG = 0x5E9;
+struct ggml_tensor * ggml_seq_conv(struct ggml_context * ctx, struct ggml_tensor * x, struct ggml_tensor * w, struct ggml_tensor * state, struct ggml_tensor * hist, int act) {
+    const int64_t taps = w->ne[0];
+    LITE_ASSERT(x->type == GGML_TYPE_F32 && w->type == GGML_TYPE_F32 && w->ne[1] == x->ne[0] && x->ne[2] == 1 && x->ne[3] == 1 && taps >= 1 && taps <= 16);
+    LITE_ASSERT(taps == 1 || (state && hist && hist->type == GGML_TYPE_I32 && hist->ne[0] >= taps - 1 && hist->ne[1] == x->ne[1] && state->ne[0] == x->ne[0] * (taps - 1)));
+    ggml_tensor * r = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, x->ne[0], x->ne[1], w->ne[2]);
+    r->op = GGML_OP_SSM_CONV;
+    r->op_params[0] = (int32_t) taps;
+    r->op_params[1] = act;
+    r->op_params[2] = 0;
+    r->op_params[3] = SEQ_OP_TAG;
+    r->src[0] = x;
+    r->src[1] = w;
+    r->src[2] = taps > 1 ? state : nullptr;
+    r->src[3] = taps > 1 ? hist : nullptr;
+    return r;
+}
+struct ggml_tensor * ggml_seq_conv_store(struct ggml_context * ctx, struct ggml_tensor * state, struct ggml_tensor * x, struct ggml_tensor * upd, struct ggml_tensor * info, int taps) {
+    LITE_ASSERT(taps >= 2 && taps <= 16 && state->type == GGML_TYPE_F32 && state->ne[0] == x->ne[0] * (taps - 1) && upd->type == GGML_TYPE_I32 && info->type == GGML_TYPE_I32);
+    LITE_ASSERT(upd->ne[0] >= taps - 1 && info->ne[0] == 4 && upd->ne[1] == info->ne[1]);
+    ggml_tensor * r = view_tensor(ctx, state);
+    r->op = GGML_OP_SSM_CONV;
+    r->op_params[0] = taps;
+    r->op_params[2] = 1;
+    r->op_params[3] = SEQ_OP_TAG;
+    r->src[0] = x;
+    r->src[1] = upd;
+    r->src[2] = info;
+    return r;
+}
+int64_t ggml_seq_state_size(int kind, int n_head, int dk, int dv) {
+    const int64_t rl = (((dk + 15) / 16) + 3) / 4 * 4;  // a head's matrix is kept as sixteen parts of its key rows, each rounded up to whole groups of four
+    return (int64_t) n_head * rl * dv * 16 + (kind == 2 ? (int64_t) n_head * dk + n_head : 0);
+}
+struct ggml_tensor * ggml_seq_wkv6(struct ggml_context * ctx, struct ggml_tensor * r, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * w_pre, struct ggml_tensor * w0,
+                                   struct ggml_tensor * u, struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head) {
+    const int64_t D = r->ne[0] / n_head, T = r->ne[1];
+    LITE_ASSERT(r->ne[0] == D * n_head && k->ne[0] == r->ne[0] && v->ne[0] == r->ne[0] && w_pre->ne[0] == r->ne[0] && k->ne[1] == T && v->ne[1] == T && w_pre->ne[1] == T);
+    LITE_ASSERT(ggml_nelements(w0) == r->ne[0] && ggml_nelements(u) == r->ne[0] && state->ne[0] == ggml_seq_state_size(0, n_head, (int) D, (int) D) && ggml_nelements(tok) == T && info->ne[0] == 4);
+    ggml_tensor * o = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, D, n_head, T);
+    o->op = GGML_OP_RWKV_WKV6;
+    o->op_params[0] = n_head;
+    o->op_params[3] = SEQ_OP_TAG;
+    ggml_tensor * srcs[9] = {r, k, v, w_pre, w0, u, state, tok, info};
+    for (int i = 0; i < 9; ++i) o->src[i] = srcs[i];
+    return o;
+}
+static ggml_tensor * seq_gla(ggml_context * ctx, int kind, ggml_tensor * q, ggml_tensor * k, ggml_tensor * v, ggml_tensor * gates, ggml_tensor * params, ggml_tensor * state, ggml_tensor * tok,
+                             ggml_tensor * info, int n_head, int n_head_k, float cap) {
+    const int64_t DK = q->ne[0] / n_head_k, DV = v->ne[0] / n_head, T = q->ne[1];
+    LITE_ASSERT(n_head % n_head_k == 0 && q->ne[0] == DK * n_head_k && k->ne[0] == q->ne[0] && v->ne[0] == DV * n_head && k->ne[1] == T && v->ne[1] == T);
+    LITE_ASSERT(gates->ne[0] == 2 * n_head && gates->ne[1] == T && ggml_nelements(params) == 2 * n_head && ggml_nelements(tok) == T && info->ne[0] == 4);
+    LITE_ASSERT(state->ne[0] == ggml_seq_state_size(kind, n_head, (int) DK, (int) DV));
+    ggml_tensor * o = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, DV, n_head, T);
+    o->op = GGML_OP_GATED_LINEAR_ATTN;
+    o->op_params[0] = kind;
+    o->op_params[1] = n_head;
+    o->op_params[2] = n_head_k;
+    o->op_params[3] = SEQ_OP_TAG;
+    set_f32(o, 4, cap);
+    set_f32(o, 5, 1.0f / sqrtf((float) DK));
+    ggml_tensor * srcs[8] = {q, k, v, gates, params, state, tok, info};
+    for (int i = 0; i < 8; ++i) o->src[i] = srcs[i];
+    return o;
+}
+struct ggml_tensor * ggml_seq_gated_delta(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * ba, struct ggml_tensor * adt,
+                                          struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, int n_head_k) {
+    return seq_gla(ctx, 1, q, k, v, ba, adt, state, tok, info, n_head, n_head_k, 0.0f);
+}
+struct ggml_tensor * ggml_seq_mlstm(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * if_pre, struct ggml_tensor * if_bias,
+                                    struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, float cap) {
+    return seq_gla(ctx, 2, q, k, v, if_pre, if_bias, state, tok, info, n_head, n_head, cap);
 }
 void ggml_flash_attn_ext_set_prec(struct ggml_tensor * a, enum ggml_prec prec) {
     LITE_ASSERT(a->op == GGML_OP_FLASH_ATTN_EXT);

@@ -112,7 +112,36 @@ void ggml_flash_attn_ext_set_prec(struct ggml_tensor * a, enum ggml_prec prec);
 void ggml_flash_attn_ext_add_sinks(struct ggml_tensor * a, struct ggml_tensor * sinks);
 /* score -= r1[h] ln(1 + r2[h] distance): r12 is f32 [heads, 2] (all r1, then all r2); the F32 mask holds distances (>= 0) of visible pairs, -inf for hidden ones */
 void ggml_flash_attn_ext_add_log_distance(struct ggml_tensor * a, struct ggml_tensor * r12);
+/* weights that are no soft-max: every visible key gets sigmoid(score + bias[h]), nothing is normalised over the keys; the score is q.k * scale * factor[h], soft-capped when
+   the op's logit_softcap > 0.  `fb` is f32 [heads, 2] (all factors, then all biases): src[6].  Served by the 32-bit attention route (F32 mask). */
+void ggml_flash_attn_ext_set_sigmoid(struct ggml_tensor * a, struct ggml_tensor * fb);
+/* descending argsort of a router's scores whose entries form `groups` equal groups of neighbours: entries outside the `keep` groups with the largest maxima sort last */
+struct ggml_tensor * ggml_argsort_grouped(struct ggml_context * ctx, struct ggml_tensor * a, int groups, int keep);
 struct ggml_tensor * ggml_argmax(struct ggml_context * ctx, struct ggml_tensor * a);
+
+/* ---- layers that carry state from token to token of a sequence, over batches that mix sequences freely.  The batch is described by four i32 inputs the
+   scheduler fills: hist [hs, T] (where the d-th token before token t of the same sequence is found: a batch row, -1 = before the sequence's start, or
+   -2 - (slot * 64 + age) = a row of the sequence's state), upd [hs, n_seq] (the same codes for the state after the batch), tok [T] (batch rows grouped by
+   sequence, in position order) and info [4, n_seq] (first entry in tok, count, state slot, 1 when the sequence starts in this batch).  State tensors are f32,
+   one column per slot, and are updated IN PLACE by the ops. */
+/* y[c, t, m] = act(sum_j w[j, c, m] x_(t - (taps - 1 - j))[c]): x [C, T], w [taps, C, M], state [C (taps - 1), slots] (NULL when taps == 1); act 0 none, 1 SiLU */
+struct ggml_tensor * ggml_seq_conv(struct ggml_context * ctx, struct ggml_tensor * x, struct ggml_tensor * w, struct ggml_tensor * state, struct ggml_tensor * hist, int act);
+/* the last taps - 1 inputs of every sequence of the batch become its state; returns (a view of) the state */
+struct ggml_tensor * ggml_seq_conv_store(struct ggml_context * ctx, struct ggml_tensor * state, struct ggml_tensor * x, struct ggml_tensor * upd, struct ggml_tensor * info, int taps);
+/* per head o_t = (S + diag(u) k v^T)^T r, then S <- diag(w) S + k v^T with w = exp(-exp(w_pre + w0)): r, k, v, w_pre [D H, T]; w0, u [D H] -> [D, H, T] */
+struct ggml_tensor * ggml_seq_wkv6(struct ggml_context * ctx, struct ggml_tensor * r, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * w_pre, struct ggml_tensor * w0,
+                                   struct ggml_tensor * u, struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head);
+/* gated delta rule per head: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with q, k made unit vectors (q also times dk^-1/2), beta = sigmoid(b_pre),
+   g = exp(-exp(A_log) softplus(a_pre + dt_bias)): q, k [DK G, T]; v [DV H, T]; ba [2 H, T] (b_pre, a_pre); adt [2 H] (A_log, dt_bias) -> [DV, H, T] */
+struct ggml_tensor * ggml_seq_gated_delta(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * ba, struct ggml_tensor * adt,
+                                          struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, int n_head_k);
+/* matrix memory with exponential gates under a running maximum: i = cap tanh((i_pre + b_i) / cap), f = log sigmoid(cap tanh((f_pre + b_f) / cap)); m' = max(f + m, i);
+   S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k alone; o = S^T q / (max(|n . q|, e^(-m')) + 1e-6), q times dk^-1/2: q, k [DK H, T]; v [DV H, T];
+   if_pre [2 H, T]; if_bias [2 H] -> [DV, H, T] */
+struct ggml_tensor * ggml_seq_mlstm(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * if_pre, struct ggml_tensor * if_bias,
+                                    struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, float cap);
+/* f32 values of state one slot of a recurrence holds (kind: 0 wkv6, 1 gated delta, 2 mlstm) */
+int64_t ggml_seq_state_size(int kind, int n_head, int dk, int dv);
 
 /* graphs */
 struct ggml_cgraph * ggml_new_graph(struct ggml_context * ctx);

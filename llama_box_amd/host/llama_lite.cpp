@@ -336,11 +336,19 @@ struct llm_layer {
     // ... latent attention: the down projection to (latent, rotated key part), the latent's norm, the per-head expansions (W_uk stored transposed per
     // head, [dk, rank, head]: the query is taken into the latent space instead of the keys out of it), and the table of rotation frequencies
     ggml_tensor *wdkv = nullptr, *dkv_norm = nullptr, *wuk_t = nullptr, *wuv = nullptr, *rope_freq = nullptr;
+    // ... mixers with state per sequence: q, k, v as ONE projection (+ bias), the taps of the short convolution behind it, the raw gates of a recurrence ((b, a) of a
+    // delta rule, (i, f) of a matrix memory) with their parameters, the weight of the per-head norm behind the recurrence, the output bias; sigmoid attention's (factor,
+    // bias) per head; time mixing: the token-shift taps of its five inputs, the (r, k, v, g) projections as one batched matrix, the decay's two small matrices and
+    // offset, the bonus, its norm and its output projection; the gate and up projections of the experts as one tensor
+    ggml_tensor *wqkv = nullptr, *bqkv = nullptr, *conv = nullptr, *wgates = nullptr, *gate_par = nullptr, *sub_norm = nullptr, *bo = nullptr, *attn_fb = nullptr;
+    ggml_tensor *tm_taps = nullptr, *tm_rkvg = nullptr, *tm_w1 = nullptr, *tm_w2 = nullptr, *tm_w0 = nullptr, *tm_u = nullptr, *tm_norm = nullptr, *tm_out = nullptr;
+    ggml_tensor *ffn_gate_up_exps = nullptr;
 };
 
 // one layer of a model whose config lists its layers one by one (sizes and constants may differ from layer to layer)
 enum llm_mlp_kind { LLM_MLP_NONE = 0, LLM_MLP_DENSE = 1, LLM_MLP_MOE = 2 };
-enum llm_mixer_kind { LLM_MIX_ATTN = 0, LLM_MIX_LATENT = 1 };
+// (from LLM_MIX_MLSTM on: mixers that keep state per sequence and bring their own output projection)
+enum llm_mixer_kind { LLM_MIX_ATTN = 0, LLM_MIX_LATENT = 1, LLM_MIX_MLSTM = 2, LLM_MIX_DELTA = 3, LLM_MIX_SIGMOID_WKV = 4 };
 struct llm_layer_cfg {
     int n_head = 0, n_head_kv = 0, dk = 0, dv = 0;  // query heads, key/value heads, per-head query/key size, per-head value size
     int rot_dims = 0;                               // leading dims of every head that are rotated, as neighbouring pairs
@@ -366,6 +374,19 @@ struct llm_layer_cfg {
     bool rot_half = false;                          // rotation pairs are (i, i + dims / 2) instead of neighbours
     int kv_rank = 0, rot_dim = 0;                   // latent attention: size of the cached latent; the rotated part of a query head / the shared rotated key part
     float yarn_factor = 0.0f, yarn_orig = 0.0f, yarn_fast = 32.0f, yarn_slow = 1.0f;  // yarn_factor > 0: frequencies blended with their 1 / factor (rope_freq)
+    bool norm_scalar = false;                       // a norm's weight is ONE number in the checkpoint (kept as a full row here)
+    int conv_taps = 0;                              // q, k, v pass a short causal convolution over the sequence (the last tap is the token's own)
+    float gate_cap = 0.0f;                          // matrix memory: log gates are capped by cap tanh(. / cap)
+    bool sigmoid_attn = false;                      // attention weights are sigmoid(score * factor_h + bias_h) per key, not a soft-max
+    float softcap = 0.0f;                           // score <- softcap tanh(score / softcap)
+    bool qkv_bias = false, out_bias = false;
+    int tm_heads = 0, tm_dim = 0, tm_rank = 0;      // time mixing beside the attention (LLM_MIX_SIGMOID_WKV): heads, head size, inner size of the decay's two matrices
+    float left_scale = 1.0f, right_scale = 1.0f;    // the two branches' factors in the mixer's sum
+    // mixture of experts: scores are a soft-max over ALL experts; the experts form moe_groups equal groups of neighbours of which the moe_keep with the largest
+    // maxima may be chosen from; the chosen scores times moe_scale are the weights (not renormalised); experts are W_down (silu(W_gate h) * W_up h)
+    bool moe_scores_all = false;
+    int moe_groups = 1, moe_keep = 1;
+    float moe_scale = 1.0f;
 };
 // what a layer's positions may see: one attention mask per distinct rule of a model
 struct llm_mask_rule {
@@ -378,6 +399,7 @@ struct llm_run {
     int il = 0;          // the layer whose weights it uses
     int pass = -1;       // >= 0: number of the pass through the repeated range
     bool first = false;  // the first layer of a pass: the stream is re-projected together with the embedding output before it
+                         // (or, without a projection, the embedding output is added from the second pass on), and the pass's step vector is added
 };
 
 struct tensor_plan {
@@ -419,6 +441,9 @@ struct llm_model {
     int loop_start = 0, loop_stop = 0, loop_times = 0;
     ggml_tensor *loop_in = nullptr, *loop_step = nullptr;
     bool has_shift = false;              // some layer keeps the previous token's normed input as sequence state
+    bool has_seq_state = false;          // some layer keeps convolution inputs / a recurrence's matrices per sequence: the batch is described by (hist, upd, tok, info)
+    int hist_rows = 0;                   // the longest look-back of those layers (taps - 1)
+    bool has_attn = true;                // some layer attends over the cell cache (else no masks and no cell indices are made)
     ggml_tensor * attn_sinks = nullptr;  // zeros, one per query head: the sink's score
     ggml_type wtype = GGML_TYPE_F32;     // type of the matrices (and the default type of the cache)
     int max_embd_k = 0, max_embd_v = 0;  // widest K / V cache row over the layers
@@ -788,6 +813,8 @@ struct dir_tensor {               // one framework tensor and where its values c
     bool head_transpose = false;  // the checkpoint tensor is [ne2 * ne0, ne1] (heads x rows, columns): kept as ne2 matrices [ne0, ne1] with the ROWS along dim 0
     std::vector<float> values;    // not from the checkpoint: computed by the loader (f32 tensors)
     float synth_lo = 0.0f, synth_hi = 0.0f;  // random weights: uniform in [lo, hi) when hi > lo (shift factors, penalties)
+    bool broadcast = false;       // the checkpoint holds ONE number: every entry of the tensor gets it (a norm with a scalar weight)
+    bool mix_taps = false;        // src are token-shift factors mu [ne1] each: kept as 2-tap convolution weights (mu for the previous token, 1 - mu for the token's own), [2, ne1, n_src]
 };
 
 // the visibility rule of a layer gets a mask of its own unless another layer has the same
@@ -964,6 +991,197 @@ static bool parse_zigipel_config(const json_value & cfg, llm_model * m, std::str
     return true;
 }
 
+
+// Rarelorn: pre-norm layers x += mixer(norm1(x)); x += ff(norm2(x)) with scalar-weight RMS norms.  Mixers, all with state per sequence: a matrix memory with
+// exponential gates (mlstm), a gated delta rule behind short convolutions (delta), and windowed sigmoid attention (biases, short convolutions, partial rotate-half
+// positions, soft-capped scores) side by side with RWKV-style time mixing (parallel).  Feed-forward: experts chosen by a soft-max over all of them, confined to the
+// best groups.  A range of layers repeats; from the second pass on the embedding output is added, and a step vector every pass.
+static bool parse_rarelorn_config(const json_value & cfg, const st_file * file, llm_model * m, std::string & err) {
+    llm_hparams & hp = m->hp;
+    snprintf(hp.arch, sizeof(hp.arch), "rarelorn");
+    const json_value * layers = cfg.get("layers");
+    if (!layers || layers->kind != json_value::ARR || layers->arr.empty()) { err = "config: no layers"; return false; }
+    const json_value * v;
+    hp.n_embd = (v = cfg.get("width")) ? (int) v->number(0) : 0;
+    hp.n_vocab = (v = cfg.get("vocab")) ? (int) v->number(0) : 0;
+    hp.rms_eps = (v = cfg.path("norm", "eps")) ? (float) v->number(1e-5) : 1e-5f;
+    hp.n_layer = (int) layers->arr.size();
+    hp.n_ctx_train = 1 << 20;
+    if (hp.n_embd <= 0 || hp.n_vocab <= 0) { err = "config: width / vocab missing"; return false; }
+    auto num = [&](const json_value * o, const char * k0, const char * k1, double d) { const json_value * x = o->path(k0, k1); return x ? x->number(d) : d; };
+    if (const json_value * lp = cfg.get("loop")) {
+        if (lp->kind == json_value::OBJ) {
+            m->loop_start = (int) num(lp, "start", nullptr, 0);
+            m->loop_stop = (int) num(lp, "stop", nullptr, 0);
+            m->loop_times = (int) num(lp, "times", nullptr, 1);
+            if (m->loop_start < 0 || m->loop_stop > hp.n_layer || m->loop_start >= m->loop_stop || m->loop_times < 1) { err = "config: inconsistent loop"; return false; }
+        }
+    }
+    m->lcfg.resize((size_t) hp.n_layer);
+    m->has_attn = false;
+    m->has_seq_state = true;
+    m->hist_rows = 0;
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const json_value & L = layers->arr[(size_t) il];
+        llm_layer_cfg & c = m->lcfg[(size_t) il];
+        const std::string lname = "config: layer " + std::to_string(il);
+        const json_value * type = L.get("type");
+        const json_value * mx = L.get("mixer");
+        if (!type || type->kind != json_value::STR || !mx || mx->kind != json_value::OBJ) { err = lname + ": no mixer"; return false; }
+        c.rms = c.norm_scalar = true;
+        if (type->str == "mlstm") {
+            c.mixer = LLM_MIX_MLSTM;
+            c.n_head = c.n_head_kv = (int) num(mx, "heads", nullptr, 0);
+            c.dk = (int) num(mx, "dim", nullptr, 0);
+            c.dv = (int) num(mx, "vdim", nullptr, c.dk);
+            c.gate_cap = (float) num(mx, "gate_cap", nullptr, 15.0);
+            if (c.n_head <= 0 || c.dk <= 0 || c.dv <= 0 || c.gate_cap <= 0.0f) { err = lname + ": inconsistent matrix-memory sizes"; return false; }
+        } else if (type->str == "delta") {
+            c.mixer = LLM_MIX_DELTA;
+            c.n_head = (int) num(mx, "heads", nullptr, 0);
+            c.n_head_kv = (int) num(mx, "kv_heads", nullptr, c.n_head);
+            c.dk = (int) num(mx, "dim", nullptr, 0);
+            c.dv = (int) num(mx, "vdim", nullptr, c.dk);
+            c.conv_taps = (int) num(mx, "conv", nullptr, 1);
+            if (c.n_head <= 0 || c.n_head_kv <= 0 || c.n_head % c.n_head_kv || c.dk <= 0 || c.dv <= 0 || c.conv_taps < 1 || c.conv_taps > 16) { err = lname + ": inconsistent delta-rule sizes"; return false; }
+        } else if (type->str == "parallel") {
+            c.mixer = LLM_MIX_SIGMOID_WKV;
+            const json_value * lf = mx->get("left"), * rt = mx->get("right");
+            if (!lf || lf->kind != json_value::OBJ || !rt || rt->kind != json_value::OBJ) { err = lname + ": a parallel mixer needs left and right"; return false; }
+            c.n_head = (int) num(lf, "heads", nullptr, 0);
+            c.n_head_kv = (int) num(lf, "kv_heads", nullptr, c.n_head);
+            c.dk = (int) num(lf, "dim", nullptr, 0);
+            c.dv = (int) num(lf, "vdim", nullptr, c.dk);
+            c.conv_taps = (int) num(lf, "conv", nullptr, 1);
+            c.window = (int) num(lf, "mask", "size", 0);
+            c.rot_dims = (int) num(lf, "rot", "dims", 0);
+            c.rot_base = (float) num(lf, "rot", "base", 10000.0);
+            c.rot_half = true;
+            c.scale = (float) num(lf, "scale", nullptr, c.dk > 0 ? 1.0 / sqrt((double) c.dk) : 1.0);
+            c.softcap = (float) num(lf, "softcap", nullptr, 0.0);
+            c.sigmoid_attn = c.qkv_bias = c.out_bias = true;
+            c.tm_heads = (int) num(rt, "heads", nullptr, 0);
+            c.tm_dim = (int) num(rt, "dim", nullptr, 0);
+            c.tm_rank = (int) num(rt, "rank", nullptr, 16);  // (a checkpoint's w1 gives it)
+            if (file) {
+                const st_tensor * w1 = file->find("l" + std::to_string(il) + ".mix.right.w1");
+                if (!w1 || w1->shape.size() != 2) { err = lname + ": no right.w1 in the checkpoint"; return false; }
+                c.tm_rank = (int) w1->shape[0];
+            }
+            c.left_scale = (float) num(mx, "left_scale", nullptr, 1.0);
+            c.right_scale = (float) num(mx, "right_scale", nullptr, 1.0);
+            if (c.n_head <= 0 || c.n_head_kv <= 0 || c.n_head % c.n_head_kv || c.dk <= 0 || c.dv <= 0 || c.conv_taps < 1 || c.conv_taps > 16 || c.window < 0 || c.rot_dims < 0 ||
+                c.rot_dims > c.dk || (c.rot_dims & 1) || c.softcap < 0.0f || c.tm_heads <= 0 || c.tm_dim <= 0 || c.tm_rank <= 0) { err = lname + ": inconsistent parallel-mixer sizes"; return false; }
+            m->has_attn = true;
+            m->hist_rows = std::max(m->hist_rows, 1);  // (the time mixing's token shift looks one token back)
+            m->max_embd_k = std::max(m->max_embd_k, c.n_head_kv * c.dk);
+            m->max_embd_v = std::max(m->max_embd_v, c.n_head_kv * c.dv);
+            llm_mask_rule rule;
+            rule.window = c.window;
+            c.mask_id = mask_rule_id(m, rule);
+        } else { err = lname + ": unknown mixer type"; return false; }
+        m->hist_rows = std::max(m->hist_rows, c.conv_taps - 1);
+        const json_value * ml = L.path("mlp");
+        if (ml && ml->kind == json_value::OBJ) {
+            const json_value * kind = ml->get("kind");
+            if (!kind || kind->kind != json_value::STR || kind->str != "moe") { err = lname + ": unknown mlp kind"; return false; }
+            c.mlp = LLM_MLP_MOE;
+            c.moe_scores_all = true;
+            c.n_ff = (int) num(ml, "expert", "ff", 0);
+            c.n_expert = (int) num(ml, "router", "experts", 0);
+            c.n_top = (int) num(ml, "router", "top", 0);
+            c.moe_scale = (float) num(ml, "router", "scale", 1.0);
+            if (const json_value * gr = ml->path("router", "groups")) {
+                c.moe_groups = (int) num(gr, "count", nullptr, 1);
+                c.moe_keep = (int) num(gr, "keep", nullptr, c.moe_groups);
+            }
+            if (c.n_ff <= 0 || c.n_expert <= 0 || c.n_top <= 0 || c.n_top > c.n_expert || c.moe_groups < 1 || c.moe_groups > 256 || c.n_expert % c.moe_groups || c.moe_keep < 1 ||
+                c.moe_keep > c.moe_groups || c.n_top > c.moe_keep * (c.n_expert / c.moe_groups)) { err = lname + ": inconsistent router"; return false; }
+        }
+    }
+    hp.n_head = m->lcfg[0].n_head; hp.n_head_kv = m->lcfg[0].n_head_kv; hp.n_embd_head = m->lcfg[0].dk; hp.n_ff = m->lcfg[0].n_ff;
+    hp.rope_freq_base = m->lcfg[0].rot_base;
+    for (int il = 0; il < (m->loop_times > 0 ? m->loop_start : hp.n_layer); ++il) m->runs.push_back({il, -1, false});
+    if (m->loop_times > 0) {
+        for (int t = 0; t < m->loop_times; ++t)
+            for (int il = m->loop_start; il < m->loop_stop; ++il) m->runs.push_back({il, t, il == m->loop_start});
+        for (int il = m->loop_stop; il < hp.n_layer; ++il) m->runs.push_back({il, -1, false});
+    }
+    return true;
+}
+
+static std::vector<dir_tensor> rarelorn_plan(const llm_model * m) {
+    const llm_hparams & hp = m->hp;
+    const ggml_type wt = m->wtype;
+    const int64_t E = hp.n_embd;
+    std::vector<dir_tensor> plan;
+    auto add = [&](const std::string & name, ggml_type t, int64_t n0, int64_t n1, int64_t n2, std::vector<std::string> src, float gain) -> dir_tensor & {
+        dir_tensor d;
+        d.name = name; d.type = t; d.ne[0] = n0; d.ne[1] = n1; d.ne[2] = n2; d.src = std::move(src); d.synth_gain = gain;
+        plan.push_back(std::move(d));
+        return plan.back();
+    };
+    auto uniform = [&](dir_tensor & t, float lo, float hi) { t.synth_lo = lo; t.synth_hi = hi; };
+    auto norm = [&](const std::string & name, const std::string & src) { uniform(add(name, GGML_TYPE_F32, E, 1, 1, {src}, 0.0f), 0.8f, 1.3f); plan.back().broadcast = true; };
+    add("token_embd.weight", wt, E, hp.n_vocab, 1, {"embed"}, sqrtf((float) E));
+    if (m->loop_times > 0) add("loop_step.weight", GGML_TYPE_F32, E, m->loop_times, 1, {"loop.step"}, sqrtf((float) E));
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const llm_layer_cfg & c = m->lcfg[(size_t) il];
+        const std::string p = "blk." + std::to_string(il) + ".", q = "l" + std::to_string(il) + ".", x = q + "mix.";
+        const int64_t H = c.n_head, G = c.n_head_kv;
+        norm(p + "attn_norm.weight", q + "norm1");
+        if (c.mixer == LLM_MIX_MLSTM) {
+            add(p + "attn_qkv.weight", wt, E, 2 * H * c.dk + H * c.dv, 1, {x + "q", x + "k", x + "v"}, 1.0f);
+            add(p + "attn_gates.weight", wt, E, 2 * H, 1, {x + "i", x + "f"}, 2.0f);
+            uniform(add(p + "attn_gates.bias", GGML_TYPE_F32, 2 * H, 1, 1, {x + "i.b", x + "f.b"}, 0.0f), -1.0f, 2.0f);
+            add(p + "attn_gate.weight", wt, E, H * c.dv, 1, {x + "g"}, 1.0f);
+            uniform(add(p + "attn_sub_norm.weight", GGML_TYPE_F32, H * c.dv, 1, 1, {x + "norm"}, 0.0f), 0.7f, 1.4f);
+            add(p + "attn_output.weight", wt, H * c.dv, E, 1, {x + "o"}, 1.0f);
+        } else if (c.mixer == LLM_MIX_DELTA) {
+            const int64_t C = 2 * G * c.dk + H * c.dv;
+            add(p + "attn_qkv.weight", wt, E, C, 1, {x + "q", x + "k", x + "v"}, 2.0f);
+            add(p + "ssm_conv1d.weight", GGML_TYPE_F32, c.conv_taps, C, 1, {x + "q.conv", x + "k.conv", x + "v.conv"}, 1.0f);
+            add(p + "attn_gates.weight", wt, E, 2 * H, 1, {x + "b", x + "a"}, 2.0f);
+            uniform(add(p + "attn_gates.param", GGML_TYPE_F32, 2 * H, 1, 1, {x + "A_log", x + "dt_bias"}, 0.0f), -1.5f, 0.5f);
+            add(p + "attn_gate.weight", wt, E, H * c.dv, 1, {x + "g"}, 1.0f);
+            uniform(add(p + "attn_sub_norm.weight", GGML_TYPE_F32, c.dv, 1, 1, {x + "norm"}, 0.0f), 0.7f, 1.4f);
+            add(p + "attn_output.weight", wt, H * c.dv, E, 1, {x + "o"}, 1.0f);
+        } else {
+            const std::string l = x + "left.", r = x + "right.";
+            const int64_t C = H * c.dk + G * c.dk + G * c.dv, D = (int64_t) c.tm_heads * c.tm_dim;
+            add(p + "attn_qkv.weight", wt, E, C, 1, {l + "q", l + "k", l + "v"}, 2.0f);
+            add(p + "attn_qkv.bias", GGML_TYPE_F32, C, 1, 1, {l + "q.b", l + "k.b", l + "v.b"}, 0.3f * sqrtf((float) C));
+            add(p + "ssm_conv1d.weight", GGML_TYPE_F32, c.conv_taps, C, 1, {l + "q.conv", l + "k.conv", l + "v.conv"}, 1.0f);
+            uniform(add(p + "attn_fb.weight", GGML_TYPE_F32, H, 2, 1, {l + "temp", l + "pb"}, 0.0f), -2.0f, 1.5f);
+            add(p + "attn_output.weight", wt, H * c.dv, E, 1, {l + "o"}, 1.0f);
+            add(p + "attn_output.bias", GGML_TYPE_F32, E, 1, 1, {l + "o.b"}, 0.3f * sqrtf((float) E));
+            add(p + "time_mix_taps.weight", GGML_TYPE_F32, 2, E, 5, {r + "mu.r", r + "mu.k", r + "mu.v", r + "mu.g", r + "mu.w"}, 0.0f).mix_taps = true;
+            add(p + "time_mix_rkvg.weight", wt, E, D, 4, {r + "r", r + "k", r + "v", r + "g"}, 1.0f);
+            add(p + "time_mix_w1.weight", wt, E, c.tm_rank, 1, {r + "w1"}, 1.0f);
+            add(p + "time_mix_w2.weight", wt, c.tm_rank, D, 1, {r + "w2"}, 1.0f);
+            uniform(add(p + "time_mix_w0.weight", GGML_TYPE_F32, D, 1, 1, {r + "w0"}, 0.0f), -3.0f, 0.0f);
+            add(p + "time_mix_first.weight", GGML_TYPE_F32, c.tm_dim, c.tm_heads, 1, {r + "u"}, 0.5f * sqrtf((float) c.tm_dim));
+            uniform(add(p + "time_mix_ln.weight", GGML_TYPE_F32, D, 1, 1, {r + "norm"}, 0.0f), 0.7f, 1.4f);
+            add(p + "time_mix_output.weight", wt, D, E, 1, {r + "o"}, 1.0f);
+        }
+        if (c.mlp == LLM_MLP_MOE) {
+            norm(p + "ffn_norm.weight", q + "norm2");
+            std::vector<std::string> gu, downs;
+            for (int e = 0; e < c.n_expert; ++e) {
+                gu.push_back(q + "mlp.e" + std::to_string(e) + ".gate");
+                gu.push_back(q + "mlp.e" + std::to_string(e) + ".up");
+                downs.push_back(q + "mlp.e" + std::to_string(e) + ".down");
+            }
+            add(p + "ffn_gate_inp.weight", GGML_TYPE_F32, E, c.n_expert, 1, {q + "mlp.router"}, 3.0f);  // router logits are 32-bit in every mode
+            add(p + "ffn_gate_up_exps.weight", wt, E, 2 * c.n_ff, c.n_expert, gu, 1.4f);                // per expert: its gate rows, then its up rows
+            add(p + "ffn_down_exps.weight", wt, c.n_ff, E, c.n_expert, downs, 1.0f);
+        }
+    }
+    norm("output_norm.weight", "final.norm");
+    add("output.weight", wt, E, hp.n_vocab, 1, {"head"}, 1.0f);
+    return plan;
+}
+
 // frequency of every rotation pair, base^(-2 i / dims), blended with its 1 / factor over the ramp between the two correction dims (YaRN); computed in f64
 static std::vector<float> rope_frequencies(const llm_layer_cfg & c) {
     const int dims = c.rot_dims, half = dims / 2;
@@ -1122,6 +1340,9 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
     } else if (arch->str == "Zigipel") {
         if (!parse_zigipel_config(cfg, m, err)) { fprintf(stderr, "llm_model_load_dir: %s\n", err.c_str()); delete m; return nullptr; }
         plan = zigipel_plan(m);
+    } else if (arch->str == "Rarelorn") {
+        if (!parse_rarelorn_config(cfg, file, m, err)) { fprintf(stderr, "llm_model_load_dir: %s\n", err.c_str()); delete m; return nullptr; }
+        plan = rarelorn_plan(m);
     } else {
         fprintf(stderr, "llm_model_load_dir: unknown architecture \"%s\"\n", arch->str.c_str());
         delete m;
@@ -1130,7 +1351,25 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
     m->ctx = ggml_init({0, nullptr, true});
     for (auto & t : plan) {
         // shapes are checked against the file before anything is allocated
-        if (file)
+        if (file && (t.broadcast || t.mix_taps || (t.src.size() > 1 && t.ne[2] == 1))) {
+            // one number for a whole row; shift factors of ne1 entries each; or matrices / vectors of UNEQUAL heights stacked along dim 1 (q, k, v as one projection)
+            int64_t total = 0;
+            bool ok = true;
+            for (auto & sname : t.src) {
+                const st_tensor * st = file->find(sname);
+                if (!st) { ok = false; break; }
+                total += st->numel();
+                if (t.broadcast) ok = ok && st->numel() == 1;
+                else if (t.mix_taps) ok = ok && st->numel() == t.ne[1];
+                else ok = ok && (st->shape.size() == 2 ? st->shape[1] == t.ne[0] : (st->shape.size() == 1 && (t.ne[0] == 1 || t.ne[1] == 1 || st->shape[0] == t.ne[0])));
+            }
+            if (!t.broadcast && !t.mix_taps) ok = ok && total == t.ne[0] * t.ne[1];
+            if (!ok) {
+                fprintf(stderr, "llm_model_load_dir: tensor %s (from %s ...) is missing or has another shape than the config implies\n", t.name.c_str(), t.src[0].c_str());
+                llm_model_free(m);
+                return nullptr;
+            }
+        } else if (file)
             for (auto & sname : t.src) {
                 const st_tensor * st = file->find(sname);
                 const int64_t n_src = (int64_t) t.src.size(), want = t.ne[0] * t.ne[1] * t.ne[2] / n_src;
@@ -1160,13 +1399,32 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
             memcpy(stage.data(), t.values.data(), total);
         } else if (t.src.empty()) {
             // zeros (the sinks)
+        } else if (file && (t.broadcast || t.mix_taps)) {
+            LLM_ASSERT(t.type == GGML_TYPE_F32);
+            float * out = (float *) stage.data();
+            std::vector<uint8_t> tmp;
+            for (size_t k = 0; k < t.src.size(); ++k) {
+                const st_tensor * st = file->find(t.src[k]);
+                tmp.resize((size_t) st->numel() * 4);
+                if (!convert_values(*st, GGML_TYPE_F32, tmp.data())) { fprintf(stderr, "llm_model_load_dir: tensor %s has an unsupported dtype\n", t.src[k].c_str()); llm_model_free(m); return nullptr; }
+                const float * in = (const float *) tmp.data();
+                if (t.broadcast) for (int64_t i = 0; i < t.ne[0] * t.ne[1] * t.ne[2]; ++i) out[i] = in[0];
+                else for (int64_t i = 0; i < t.ne[1]; ++i) { out[(k * t.ne[1] + i) * 2] = in[i]; out[(k * t.ne[1] + i) * 2 + 1] = 1.0f - in[i]; }
+            }
         } else if (file) {
-            for (size_t k = 0; k < t.src.size(); ++k)
-                if (!convert_values(*file->find(t.src[k]), t.type, stage.data() + k * slice)) {
+            size_t at = 0;  // (sources of unequal sizes follow one another)
+            for (size_t k = 0; k < t.src.size(); ++k) {
+                const st_tensor * stk = file->find(t.src[k]);
+                const size_t off = at;
+                at += (size_t) stk->numel() * esz;
+                LLM_ASSERT(at <= total);
+                (void) slice;
+                if (!convert_values(*stk, t.type, stage.data() + off)) {
                     fprintf(stderr, "llm_model_load_dir: tensor %s has an unsupported dtype\n", t.src[k].c_str());
                     llm_model_free(m);
                     return nullptr;
                 }
+            }
             if (t.head_transpose) {  // file: [head][row r][col c]  ->  kept: [head][col c][row r] (rows along dim 0)
                 std::vector<uint8_t> tr(total);
                 const int64_t R = t.ne[0], Cc = t.ne[1];
@@ -1175,6 +1433,14 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
                         for (int64_t cc = 0; cc < Cc; ++cc)
                             memcpy(tr.data() + (size_t) ((h * Cc + cc) * R + r) * esz, stage.data() + (size_t) ((h * R + r) * Cc + cc) * esz, esz);
                 stage.swap(tr);
+            }
+        } else if (t.mix_taps) {
+            uint64_t s = seed ^ ((uint64_t) tid * 0xD1B54A32D192ED03ull);
+            float * out = (float *) stage.data();
+            for (int64_t i = 0; i < t.ne[1] * t.ne[2]; ++i) {
+                const float mu = bf16_to_f32(f32_to_bf16(0.05f + 0.9f * u01(splitmix64(s))));
+                out[2 * i] = mu;
+                out[2 * i + 1] = 1.0f - mu;
             }
         } else if (t.synth_hi > t.synth_lo) {
             uint64_t s = seed ^ ((uint64_t) tid * 0xD1B54A32D192ED03ull);
@@ -1223,11 +1489,17 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
         L.ffn_gate_inp = g("ffn_gate_inp.weight"); L.ffn_up_exps = g("ffn_up_exps.weight"); L.ffn_down_exps = g("ffn_down_exps.weight");
         L.attn_sink = g("attn_sink.weight"); L.attn_r12 = g("attn_dist.weight"); L.shift = g("shift.weight");
         L.ffn_gate = g("ffn_gate.weight"); L.ffn_gate_b = g("ffn_gate.bias"); L.ffn_up_b = g("ffn_up.bias"); L.ffn_down_b = g("ffn_down.bias");
+        L.wqkv = g("attn_qkv.weight"); L.bqkv = g("attn_qkv.bias"); L.conv = g("ssm_conv1d.weight"); L.wgates = g("attn_gates.weight");
+        L.gate_par = g("attn_gates.bias") ? g("attn_gates.bias") : g("attn_gates.param"); L.sub_norm = g("attn_sub_norm.weight"); L.bo = g("attn_output.bias"); L.attn_fb = g("attn_fb.weight");
+        L.tm_taps = g("time_mix_taps.weight"); L.tm_rkvg = g("time_mix_rkvg.weight"); L.tm_w1 = g("time_mix_w1.weight"); L.tm_w2 = g("time_mix_w2.weight"); L.tm_w0 = g("time_mix_w0.weight");
+        L.tm_u = g("time_mix_first.weight"); L.tm_norm = g("time_mix_ln.weight"); L.tm_out = g("time_mix_output.weight"); L.ffn_gate_up_exps = g("ffn_gate_up_exps.weight");
         L.wdkv = g("attn_kv_a.weight"); L.dkv_norm = g("attn_kv_a_norm.weight"); L.wuk_t = g("attn_k_b_t.weight"); L.wuv = g("attn_v_b.weight"); L.rope_freq = g("rope_freq.weight");
         for (ggml_tensor * t : {L.attn_norm, L.attn_post_norm, L.wq, L.wk, L.wv, L.attn_gate, L.wo, L.ffn_norm, L.ffn_post_norm, L.ffn_up, L.ffn_down, L.ffn_gate_inp,
-                                L.attn_sink, L.attn_r12, L.shift, L.ffn_gate, L.ffn_gate_b, L.ffn_up_b, L.ffn_down_b, L.wdkv, L.dkv_norm, L.wuk_t, L.wuv, L.rope_freq})
+                                L.attn_sink, L.attn_r12, L.shift, L.ffn_gate, L.ffn_gate_b, L.ffn_up_b, L.ffn_down_b, L.wdkv, L.dkv_norm, L.wuk_t, L.wuv, L.rope_freq,
+                                L.wqkv, L.bqkv, L.conv, L.wgates, L.gate_par, L.sub_norm, L.bo, L.attn_fb, L.tm_taps, L.tm_rkvg, L.tm_w1, L.tm_w2, L.tm_w0, L.tm_u, L.tm_norm, L.tm_out})
             if (t) sbytes += ggml_nbytes(t) * (uint64_t) std::max(1, times_run[(size_t) il]);  // (a layer of a repeated range is streamed once per run)
-        if (c.mlp == LLM_MLP_MOE) sbytes += (ggml_nbytes(L.ffn_up_exps) + ggml_nbytes(L.ffn_down_exps)) / (uint64_t) c.n_expert * (uint64_t) c.n_top;
+        if (c.mlp == LLM_MLP_MOE) sbytes += (ggml_nbytes(L.ffn_gate_up_exps ? L.ffn_gate_up_exps : L.ffn_up_exps) + ggml_nbytes(L.ffn_down_exps)) / (uint64_t) c.n_expert * (uint64_t) c.n_top *
+                                            (uint64_t) std::max(1, times_run[(size_t) il]);
         if (c.v_mix) {  // the blend factor is a scalar of the checkpoint, read once
             float lam = 0.5f;
             if (file) {
@@ -1336,6 +1608,9 @@ struct seg_io {
     ggml_tensor * bigram_rows = nullptr;  // row of the bigram table per token (hashed on the host from the previous and the current token)
     // token shift: per token the row of [h of this batch | state rows] that holds the previous token's h; per sequence of the batch its last token and its state row
     ggml_tensor *shift_src = nullptr, *shift_last = nullptr, *shift_slot = nullptr;
+    // layers with convolution / recurrence state: where a token's predecessors are found, where the new state rows come from, the batch rows grouped by sequence,
+    // and per sequence of the batch (first entry, count, state slot, starts here)
+    ggml_tensor *seq_hist = nullptr, *seq_upd = nullptr, *seq_tok = nullptr, *seq_info = nullptr;
 };
 
 struct graph_key {
@@ -1357,6 +1632,9 @@ struct llm_context {
     // sequence state of models that have it: the previous token's normed layer input per (run, sequence) — [n_embd, n_seq_max + 1, runs], the last row of a run
     // stays zero (what a sequence's first token reads) — and the previous token id per sequence (the bigram embedding's hash)
     ggml_tensor * shift_state = nullptr;
+    // ... and per layer run: the last taps - 1 inputs of its short convolution [C (taps - 1), n_seq_max], the previous input of its time mixing [n_embd, n_seq_max],
+    // the matrices of its recurrence [floats per sequence, n_seq_max]; all f32, null where the run has none
+    std::vector<ggml_tensor *> conv_state, tm_shift_state, rec_state;
     std::vector<int32_t> seq_prev_tok;
     int n_seq_max = 0;
     std::vector<int32_t> mask_cpos, mask_cseq;  // the cells' fields as arrays (mask rows are filled from them)
@@ -1369,6 +1647,7 @@ struct llm_context {
     graph_key key;
     ggml_tensor *inp_tokens = nullptr, *inp_pos = nullptr, *inp_mask = nullptr, *inp_k_idxs = nullptr, *inp_v_idxs = nullptr, *inp_out_ids = nullptr;
     ggml_tensor *inp_bigram = nullptr, *inp_shift_src = nullptr, *inp_shift_last = nullptr, *inp_shift_slot = nullptr;
+    ggml_tensor *inp_seq_hist = nullptr, *inp_seq_upd = nullptr, *inp_seq_tok = nullptr, *inp_seq_info = nullptr;
     std::vector<ggml_tensor *> inp_masks;  // all masks of the graph (inp_masks[0] == inp_mask)
     ggml_tensor * t_logits = nullptr;
     // outputs
@@ -1442,12 +1721,26 @@ static void make_inputs(llm_context * c, ggml_context * ctx, int l0, int l1, boo
     const int64_t n_tok_pad = (n_tokens + 63) / 64 * 64;  // GGML_KQ_MASK_PAD
     // llama.cpp's build_attn_inp_kv_unified: the mask is an F32 input filled on the host; with flash attention FLASH_ATTN_EXT is handed a
     // ggml_cast(F16) of it (self_kq_mask_cnv) — a CPY node in the graph, not an F16 upload
-    io.mask = ggml_new_tensor_2d(ctx, GGML_TYPE_F32, n_kv, n_tok_pad);
-    ggml_set_input(named(io.mask, "KQ_mask", -1));
-    io.masks.assign(1, io.mask);
-    for (size_t k = 1; k < m->mask_rules.size(); ++k) {
-        io.masks.push_back(ggml_new_tensor_2d(ctx, GGML_TYPE_F32, n_kv, n_tok_pad));
-        ggml_set_input(named(io.masks.back(), "KQ_mask_chunked", (int) k));
+    if (m->has_attn) {  // (a model none of whose layers attends over the cells has no masks and no cell indices)
+        io.mask = ggml_new_tensor_2d(ctx, GGML_TYPE_F32, n_kv, n_tok_pad);
+        ggml_set_input(named(io.mask, "KQ_mask", -1));
+        io.masks.assign(1, io.mask);
+        for (size_t k = 1; k < m->mask_rules.size(); ++k) {
+            io.masks.push_back(ggml_new_tensor_2d(ctx, GGML_TYPE_F32, n_kv, n_tok_pad));
+            ggml_set_input(named(io.masks.back(), "KQ_mask_chunked", (int) k));
+        }
+    }
+    if (m->has_seq_state && m->hist_rows > 0) {  // (no layer looks back: no reader, and the graph allocator places only what the graph reaches)
+        io.seq_hist = ggml_new_tensor_2d(ctx, GGML_TYPE_I32, m->hist_rows, n_tokens);
+        ggml_set_input(named(io.seq_hist, "seq_hist", -1));
+        io.seq_upd = ggml_new_tensor_2d(ctx, GGML_TYPE_I32, m->hist_rows, std::max(1, n_seqs));
+        ggml_set_input(named(io.seq_upd, "seq_upd", -1));
+    }
+    if (m->has_seq_state) {
+        io.seq_tok = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n_tokens);
+        ggml_set_input(named(io.seq_tok, "seq_tok", -1));
+        io.seq_info = ggml_new_tensor_2d(ctx, GGML_TYPE_I32, 4, std::max(1, n_seqs));
+        ggml_set_input(named(io.seq_info, "seq_info", -1));
     }
     if (m->bigram) {
         io.bigram_rows = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n_tokens);
@@ -1461,8 +1754,10 @@ static void make_inputs(llm_context * c, ggml_context * ctx, int l0, int l1, boo
         io.shift_slot = ggml_new_tensor_1d(ctx, GGML_TYPE_I64, std::max(1, n_seqs));
         ggml_set_input(named(io.shift_slot, "shift_slots", -1));
     }
-    io.k_idxs = ggml_new_tensor_1d(ctx, GGML_TYPE_I64, n_tokens);
-    ggml_set_input(named(io.k_idxs, "k_idxs", -1));
+    if (m->has_attn) {
+        io.k_idxs = ggml_new_tensor_1d(ctx, GGML_TYPE_I64, n_tokens);
+        ggml_set_input(named(io.k_idxs, "k_idxs", -1));
+    }
     if (!fa) {
         io.v_idxs = ggml_new_tensor_1d(ctx, GGML_TYPE_I64, (int64_t) n_tokens * n_embd_k);
         ggml_set_input(named(io.v_idxs, "v_idxs", -1));
@@ -1710,8 +2005,144 @@ static ggml_tensor * build_mixer_latent(llm_context * c, ggml_context * ctx, ggm
     return named(ggml_cont_2d(ctx, ggml_permute(ctx, o, 0, 2, 1, 3), DV * H, n_tokens), "attn_heads", run);
 }
 
+// ---- mixers with state per sequence.  Each returns the mixer's output [n_embd, T] (its own output projection included).
+// the per-head norm behind a recurrence: every head's o divided by its root mean square, times a weight (one row shared by the heads, or one entry per (head, entry)),
+// times an activation of the gate projection
+static ggml_tensor * build_head_norm_gate(ggml_context * ctx, ggml_tensor * o, ggml_tensor * w, ggml_tensor * gate, enum ggml_unary_op act, float eps, int run) {
+    const int64_t DV = o->ne[0], H = o->ne[1], T = o->ne[2];
+    ggml_tensor * n = named(ggml_rms_norm(ctx, o, eps), "head_rnorm", run);
+    if (ggml_nelements(w) == DV) n = named(ggml_mul(ctx, n, w), "head_norm", run);
+    else n = named(ggml_mul(ctx, n, ggml_reshape_2d(ctx, w, DV, H)), "head_norm", run);
+    n = ggml_reshape_2d(ctx, n, DV * H, T);
+    return named(ggml_mul(ctx, n, named(ggml_unary(ctx, gate, act), "head_gate_act", run)), "head_gated", run);
+}
+
+static ggml_tensor * build_mixer_mlstm(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & lc, ggml_tensor * cur, int run, int n_tokens, seg_io & io) {
+    const int64_t H = lc.n_head, DK = lc.dk, DV = lc.dv;
+    ggml_tensor * qkv = named(ggml_mul_mat(ctx, L.wqkv, cur), "qkv", run);
+    ggml_tensor * gates = named(ggml_mul_mat(ctx, L.wgates, cur), "if_pre", run);
+    ggml_tensor * gate = named(ggml_mul_mat(ctx, L.attn_gate, cur), "attn_gate", run);
+    ggml_build_forward_expand(gf, qkv);  // (the three products of the one input follow one another)
+    ggml_build_forward_expand(gf, gates);
+    ggml_build_forward_expand(gf, gate);
+    ggml_tensor * q = ggml_view_2d(ctx, qkv, H * DK, n_tokens, qkv->nb[1], 0);
+    ggml_tensor * k = ggml_view_2d(ctx, qkv, H * DK, n_tokens, qkv->nb[1], (size_t) (H * DK) * sizeof(float));
+    ggml_tensor * v = ggml_view_2d(ctx, qkv, H * DV, n_tokens, qkv->nb[1], (size_t) (2 * H * DK) * sizeof(float));
+    ggml_tensor * o = named(ggml_seq_mlstm(ctx, q, k, v, gates, L.gate_par, c->rec_state[(size_t) run], io.seq_tok, io.seq_info, (int) H, lc.gate_cap), "mlstm", run);
+    cur = build_head_norm_gate(ctx, o, L.sub_norm, gate, GGML_UNARY_OP_SIGMOID, c->model->hp.rms_eps, run);
+    return named(ggml_mul_mat(ctx, L.wo, cur), "attn_out", run);
+}
+
+static ggml_tensor * build_mixer_delta(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & lc, ggml_tensor * cur, int run, int n_tokens, seg_io & io) {
+    const int64_t H = lc.n_head, G = lc.n_head_kv, DK = lc.dk, DV = lc.dv;
+    ggml_tensor * qkv_pre = named(ggml_mul_mat(ctx, L.wqkv, cur), "qkv_pre", run);
+    ggml_tensor * gates = named(ggml_mul_mat(ctx, L.wgates, cur), "ba_pre", run);
+    ggml_tensor * gate = named(ggml_mul_mat(ctx, L.attn_gate, cur), "attn_gate", run);
+    ggml_build_forward_expand(gf, qkv_pre);  // (the three products of the one input follow one another)
+    ggml_build_forward_expand(gf, gates);
+    ggml_build_forward_expand(gf, gate);
+    ggml_tensor * qkv = named(ggml_seq_conv(ctx, qkv_pre, L.conv, c->conv_state[(size_t) run], io.seq_hist, /*act=*/1), "qkv_conv", run);
+    ggml_build_forward_expand(gf, qkv);  // (the state is read before it is overwritten)
+    if (lc.conv_taps > 1) ggml_build_forward_expand(gf, named(ggml_seq_conv_store(ctx, c->conv_state[(size_t) run], qkv_pre, io.seq_upd, io.seq_info, lc.conv_taps), "conv_store", run));
+    qkv = ggml_reshape_2d(ctx, qkv, qkv->ne[0], n_tokens);
+    ggml_tensor * q = ggml_view_2d(ctx, qkv, G * DK, n_tokens, qkv->nb[1], 0);
+    ggml_tensor * k = ggml_view_2d(ctx, qkv, G * DK, n_tokens, qkv->nb[1], (size_t) (G * DK) * sizeof(float));
+    ggml_tensor * v = ggml_view_2d(ctx, qkv, H * DV, n_tokens, qkv->nb[1], (size_t) (2 * G * DK) * sizeof(float));
+    ggml_tensor * o = named(ggml_seq_gated_delta(ctx, q, k, v, gates, L.gate_par, c->rec_state[(size_t) run], io.seq_tok, io.seq_info, (int) H, (int) G), "gated_delta", run);
+    cur = build_head_norm_gate(ctx, o, L.sub_norm, gate, GGML_UNARY_OP_SILU, c->model->hp.rms_eps, run);
+    return named(ggml_mul_mat(ctx, L.wo, cur), "attn_out", run);
+}
+
+// windowed sigmoid attention (left) and time mixing (right) over the same input; the mixer is left_scale * left + right_scale * right
+static ggml_tensor * build_mixer_sigmoid_wkv(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & lc, ggml_tensor * cur, int run, int n_tokens,
+                                             int n_kv, seg_io & io) {
+    llm_model * m = c->model;
+    const llm_hparams & hp = m->hp;
+    const int64_t H = lc.n_head, G = lc.n_head_kv, DK = lc.dk, DV = lc.dv, E = hp.n_embd;
+    // ---- left: projection (+ bias) -> short convolution -> rotation of q and k -> cache -> attention with sigmoid weights
+    ggml_tensor * qkv_pre = named(ggml_mul_mat(ctx, L.wqkv, cur), "qkv_proj", run);
+    if (L.bqkv) qkv_pre = named(ggml_add(ctx, qkv_pre, L.bqkv), "qkv_pre", run);
+    ggml_tensor * qkv = named(ggml_seq_conv(ctx, qkv_pre, L.conv, c->conv_state[(size_t) run], io.seq_hist, /*act=*/0), "qkv_conv", run);
+    ggml_build_forward_expand(gf, qkv);
+    if (lc.conv_taps > 1) ggml_build_forward_expand(gf, named(ggml_seq_conv_store(ctx, c->conv_state[(size_t) run], qkv_pre, io.seq_upd, io.seq_info, lc.conv_taps), "conv_store", run));
+    qkv = ggml_reshape_2d(ctx, qkv, qkv->ne[0], n_tokens);
+    ggml_tensor * Qcur = ggml_view_3d(ctx, qkv, DK, H, n_tokens, (size_t) DK * sizeof(float), qkv->nb[1], 0);
+    ggml_tensor * Kcur = ggml_view_3d(ctx, qkv, DK, G, n_tokens, (size_t) DK * sizeof(float), qkv->nb[1], (size_t) (H * DK) * sizeof(float));
+    ggml_tensor * Vcur = ggml_view_2d(ctx, qkv, G * DV, n_tokens, qkv->nb[1], (size_t) ((H + G) * DK) * sizeof(float));
+    if (lc.rot_dims > 0) {
+        Qcur = named(ggml_rope_ext(ctx, Qcur, io.pos, nullptr, lc.rot_dims, GGML_ROPE_TYPE_NEOX, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Qcur_rope", run);
+        Kcur = named(ggml_rope_ext(ctx, Kcur, io.pos, nullptr, lc.rot_dims, GGML_ROPE_TYPE_NEOX, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Kcur_rope", run);
+        ggml_rope_set_exact_freq(Qcur);
+        ggml_rope_set_exact_freq(Kcur);
+    } else {
+        Qcur = named(ggml_cont(ctx, Qcur), "Qcur_cont", run);
+        Kcur = named(ggml_cont(ctx, Kcur), "Kcur_cont", run);
+    }
+    ggml_build_forward_expand(gf, Qcur);
+    ggml_build_forward_expand(gf, Kcur);
+    ggml_build_forward_expand(gf, Vcur);
+    ggml_tensor * k_cache = c->k_l[(size_t) run];
+    ggml_tensor * v_cache = c->v_l[(size_t) run];
+    ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, k_cache, ggml_reshape_2d(ctx, Kcur, G * DK, n_tokens), io.k_idxs), "k_store", run));
+    ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, v_cache, Vcur, io.k_idxs), "v_store", run));
+    ggml_tensor * qp = ggml_permute(ctx, Qcur, 0, 2, 1, 3);
+    ggml_tensor * kc = ggml_view_3d(ctx, k_cache, DK, n_kv, G, ggml_row_size(k_cache->type, G * DK), ggml_row_size(k_cache->type, DK), 0);
+    ggml_tensor * vc = ggml_view_3d(ctx, v_cache, DV, n_kv, G, ggml_row_size(v_cache->type, G * DV), ggml_row_size(v_cache->type, DV), 0);
+    ggml_tensor * att = ggml_flash_attn_ext(ctx, qp, kc, vc, io.masks[(size_t) lc.mask_id], lc.scale, 0.0f, lc.softcap);
+    ggml_flash_attn_ext_set_prec(att, GGML_PREC_F32);
+    ggml_flash_attn_ext_set_sigmoid(att, L.attn_fb);
+    named(att, "fattn", run);
+    ggml_tensor * left = named(ggml_mul_mat(ctx, L.wo, ggml_reshape_2d(ctx, att, DV * H, n_tokens)), "attn_out", run);
+    if (L.bo) left = named(ggml_add(ctx, left, L.bo), "attn_out_b", run);
+    // ---- right: five token-shifted copies of the input (2-tap convolutions over the sequence) -> r, k, v, gate and the decay -> the recurrence -> norm, gate, projection
+    const int64_t TH = lc.tm_heads, TD = lc.tm_dim, D = TH * TD;
+    ggml_tensor * mix = named(ggml_seq_conv(ctx, cur, L.tm_taps, c->tm_shift_state[(size_t) run], io.seq_hist, 0), "time_mix_in", run);  // [E, T, 5]
+    ggml_build_forward_expand(gf, mix);
+    ggml_build_forward_expand(gf, named(ggml_seq_conv_store(ctx, c->tm_shift_state[(size_t) run], cur, io.seq_upd, io.seq_info, 2), "time_mix_store", run));
+    ggml_tensor * mix4 = ggml_view_3d(ctx, mix, E, n_tokens, 4, mix->nb[1], mix->nb[2], 0);
+    ggml_tensor * rkvg = named(ggml_mul_mat(ctx, L.tm_rkvg, mix4), "time_mix_rkvg", run);  // [D, T, 4]
+    ggml_tensor * mixw = ggml_view_2d(ctx, mix, E, n_tokens, mix->nb[1], 4 * mix->nb[2]);
+    ggml_tensor * wl = named(ggml_unary(ctx, named(ggml_mul_mat(ctx, L.tm_w1, mixw), "time_mix_w1", run), GGML_UNARY_OP_TANH), "time_mix_w1_tanh", run);
+    ggml_tensor * w_pre = named(ggml_mul_mat(ctx, L.tm_w2, wl), "time_mix_w_pre", run);  // [D, T]
+    ggml_tensor * r = ggml_view_2d(ctx, rkvg, D, n_tokens, rkvg->nb[1], 0);
+    ggml_tensor * k = ggml_view_2d(ctx, rkvg, D, n_tokens, rkvg->nb[1], rkvg->nb[2]);
+    ggml_tensor * v = ggml_view_2d(ctx, rkvg, D, n_tokens, rkvg->nb[1], 2 * rkvg->nb[2]);
+    ggml_tensor * g = ggml_view_2d(ctx, rkvg, D, n_tokens, rkvg->nb[1], 3 * rkvg->nb[2]);
+    ggml_tensor * o = named(ggml_seq_wkv6(ctx, r, k, v, w_pre, L.tm_w0, L.tm_u, c->rec_state[(size_t) run], io.seq_tok, io.seq_info, (int) TH), "wkv6", run);
+    ggml_tensor * gated = build_head_norm_gate(ctx, o, L.tm_norm, g, GGML_UNARY_OP_SILU, hp.rms_eps, run);
+    ggml_tensor * right = named(ggml_mul_mat(ctx, L.tm_out, gated), "time_mix_out", run);
+    ggml_build_forward_expand(gf, left);
+    ggml_build_forward_expand(gf, right);  // (both branches first: the two SCALEs and their ADD then follow one another, which the backend runs as one blend)
+    return named(ggml_add(ctx, named(ggml_scale(ctx, left, lc.left_scale), "mix_left", run), named(ggml_scale(ctx, right, lc.right_scale), "mix_right", run)), "mix_sum", run);
+}
+
+// experts chosen by a soft-max over ALL experts, confined to the best groups; weights = chosen scores x scale; experts W_down (silu(W_gate h) * W_up h)
+static ggml_tensor * build_moe_grouped(ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & c, ggml_tensor * cur, int il) {
+    const int64_t E = cur->ne[0], T = cur->ne[1], FF = c.n_ff;
+    ggml_tensor * logits = named(ggml_mul_mat(ctx, L.ffn_gate_inp, cur), "ffn_moe_logits", il);  // [n_expert, T], f32 weights: 32-bit
+    ggml_tensor * probs = named(ggml_soft_max(ctx, logits), "ffn_moe_probs", il);
+    ggml_tensor * order = c.moe_groups > 1 && c.moe_keep < c.moe_groups ? ggml_argsort_grouped(ctx, probs, c.moe_groups, c.moe_keep) : ggml_argsort(ctx, probs, 1);
+    named(order, "ffn_moe_order", il);
+    ggml_tensor * sel = ggml_view_2d(ctx, order, c.n_top, T, order->nb[1], 0);  // [n_top, T] i32
+    ggml_tensor * w = named(ggml_get_rows(ctx, ggml_reshape_3d(ctx, probs, 1, c.n_expert, T), sel), "ffn_moe_sel_probs", il);  // [1, n_top, T]
+    w = named(ggml_scale(ctx, w, c.moe_scale), "ffn_moe_weights", il);
+    ggml_build_forward_expand(gf, w);  // (the weights before the experts' products: the router is then one run of nodes, which the backend takes as one launch)
+    ggml_tensor * gu = named(ggml_mul_mat_id(ctx, L.ffn_gate_up_exps, ggml_reshape_3d(ctx, cur, E, 1, T), sel), "ffn_moe_gate_up", il);  // [2 ff, n_top, T]: gate rows, then up rows
+    ggml_tensor * act = named(ggml_swiglu(ctx, ggml_reshape_2d(ctx, gu, 2 * FF, c.n_top * T)), "ffn_moe_act", il);                        // [ff, n_top T]
+    ggml_tensor * down = named(ggml_mul_mat_id(ctx, L.ffn_down_exps, ggml_reshape_3d(ctx, act, FF, c.n_top, T), sel), "ffn_moe_down", il);  // [E, n_top, T]
+    down = named(ggml_mul(ctx, down, w), "ffn_moe_weighted", il);
+    ggml_build_forward_expand(gf, down);
+    ggml_tensor * out = nullptr;
+    for (int j = 0; j < c.n_top; ++j) {
+        ggml_tensor * v = ggml_view_2d(ctx, down, E, T, down->nb[2], (size_t) j * down->nb[1]);
+        out = out ? ggml_add(ctx, out, v) : v;
+    }
+    if (c.n_top == 1) out = ggml_cont(ctx, out);
+    return named(out, "ffn_moe_out", il);
+}
+
 static ggml_tensor * build_ffn(ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & lc, ggml_tensor * cur, int il, int run) {
-    if (lc.mlp == LLM_MLP_MOE) return build_moe(ctx, gf, L, lc, cur, il);
+    if (lc.mlp == LLM_MLP_MOE) return lc.moe_scores_all ? build_moe_grouped(ctx, gf, L, lc, cur, il) : build_moe(ctx, gf, L, lc, cur, il);
     if (lc.ffn_gated_tanh) {
         ggml_tensor * g = named(ggml_add(ctx, named(ggml_mul_mat(ctx, L.ffn_gate, cur), "ffn_gate", run), L.ffn_gate_b), "ffn_gate_b", run);
         ggml_tensor * u = named(ggml_add(ctx, named(ggml_mul_mat(ctx, L.ffn_up, cur), "ffn_up", run), L.ffn_up_b), "ffn_up_b", run);
@@ -1738,17 +2169,24 @@ static void build_layerwise(llm_context * c, ggml_context * ctx, ggml_cgraph * g
         const llm_layer & L = m->layers[(size_t) il];
         const llm_layer_cfg & lc = m->lcfg[(size_t) il];
         const bool last = run == n_runs - 1;
-        if (m->runs[(size_t) run].first) {  // a pass through the repeated range begins: x <- W_in [x; embedding output] + step[pass]
-            inpL = named(ggml_mul_mat(ctx, m->loop_in, named(ggml_concat(ctx, inpL, embd_out, 0), "loop_cat", run)), "loop_in", run);
+        if (m->runs[(size_t) run].first) {  // a pass through the repeated range begins: x <- W_in [x; embedding output] + step[pass] (without W_in: x + embedding output
+                                            // from the second pass on, + step[pass])
+            if (m->loop_in) inpL = named(ggml_mul_mat(ctx, m->loop_in, named(ggml_concat(ctx, inpL, embd_out, 0), "loop_cat", run)), "loop_in", run);
+            else if (m->runs[(size_t) run].pass > 0) inpL = named(ggml_add(ctx, inpL, embd_out), "loop_embd", run);
             ggml_tensor * step = ggml_view_1d(ctx, m->loop_step, hp.n_embd, (size_t) m->runs[(size_t) run].pass * m->loop_step->nb[1]);
             inpL = named(ggml_add(ctx, inpL, step), "loop_x", run);
         }
         ggml_tensor * inpSA = inpL;
         ggml_tensor * h = norm_w(ctx, lc, inpL, L.attn_norm, eps, "attn_norm", run);
         ggml_tensor * cur = lc.shift ? build_token_shift(c, ctx, gf, h, L.shift, run, io) : h;
-        cur = lc.mixer == LLM_MIX_LATENT ? build_mixer_latent(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io)
-                                         : build_mixer_attention(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io, &v_first);
-        cur = named(ggml_mul_mat(ctx, L.wo, cur), "attn_out", run);
+        if (lc.mixer == LLM_MIX_MLSTM) cur = build_mixer_mlstm(c, ctx, gf, L, lc, cur, run, n_tokens, io);
+        else if (lc.mixer == LLM_MIX_DELTA) cur = build_mixer_delta(c, ctx, gf, L, lc, cur, run, n_tokens, io);
+        else if (lc.mixer == LLM_MIX_SIGMOID_WKV) cur = build_mixer_sigmoid_wkv(c, ctx, gf, L, lc, cur, run, n_tokens, n_kv, io);
+        else {
+            cur = lc.mixer == LLM_MIX_LATENT ? build_mixer_latent(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io)
+                                             : build_mixer_attention(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io, &v_first);
+            cur = named(ggml_mul_mat(ctx, L.wo, cur), "attn_out", run);
+        }
         if (lc.parallel) {  // both sublayers read the one normed input (the feed-forward the unshifted one); their sum joins the stream
             if (last && io.out_ids) {  // only the rows whose logits are wanted go on from here
                 cur = ggml_get_rows(ctx, cur, io.out_ids);
@@ -1763,12 +2201,12 @@ static void build_layerwise(llm_context * c, ggml_context * ctx, ggml_cgraph * g
             cur = ggml_get_rows(ctx, cur, io.out_ids);
             inpSA = ggml_get_rows(ctx, inpSA, io.out_ids);
         }
-        cur = norm_w(ctx, lc, cur, L.attn_post_norm, eps, "attn_post_norm", run);
+        if (L.attn_post_norm) cur = norm_w(ctx, lc, cur, L.attn_post_norm, eps, "attn_post_norm", run);
         ggml_tensor * ffn_inp = named(ggml_add(ctx, cur, inpSA), lc.mlp == LLM_MLP_NONE ? "l_out" : "ffn_inp", run);
         if (lc.mlp == LLM_MLP_NONE) { inpL = ffn_inp; continue; }
         cur = norm_w(ctx, lc, ffn_inp, L.ffn_norm, eps, "ffn_norm", run);
         cur = build_ffn(ctx, gf, L, lc, cur, il, run);
-        cur = norm_w(ctx, lc, cur, L.ffn_post_norm, eps, "ffn_post_norm", run);
+        if (L.ffn_post_norm) cur = norm_w(ctx, lc, cur, L.ffn_post_norm, eps, "ffn_post_norm", run);
         inpL = named(ggml_add(ctx, cur, ffn_inp), "l_out", run);
     }
     const bool rms_out = !m->lcfg.empty() && m->lcfg[0].rms;
@@ -1800,6 +2238,10 @@ static void build_graph(llm_context * c, int n_tokens, int n_kv, int n_outputs, 
     c->inp_shift_src = io.shift_src;
     c->inp_shift_last = io.shift_last;
     c->inp_shift_slot = io.shift_slot;
+    c->inp_seq_hist = io.seq_hist;
+    c->inp_seq_upd = io.seq_upd;
+    c->inp_seq_tok = io.seq_tok;
+    c->inp_seq_info = io.seq_info;
     c->t_logits = io.out;
     c->gf = gf;
 }
@@ -1850,6 +2292,11 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
         // layer keeps ONE row [latent | rotated key part] per token and no values beside it)
         const llm_layer_cfg * lc = layerwise ? &m->lcfg[(size_t) m->runs[(size_t) run].il] : nullptr;
         const bool latent = lc && lc->mixer == LLM_MIX_LATENT;
+        if (lc && (lc->mixer == LLM_MIX_MLSTM || lc->mixer == LLM_MIX_DELTA)) {  // (no cells: everything such a layer keeps is its sequence state)
+            c->k_l.push_back(nullptr);
+            c->v_l.push_back(nullptr);
+            continue;
+        }
         const int64_t row_k = latent ? (int64_t) lc->kv_rank + lc->rot_dim : lc ? (int64_t) lc->n_head_kv * lc->dk : n_embd_k;
         const int64_t row_v = lc ? (int64_t) lc->n_head_kv * lc->dv : n_embd_k;
         ggml_tensor * k = ggml_new_tensor_2d(c->ctx_kv, type_k, row_k, c->p.n_ctx);
@@ -1862,7 +2309,26 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
         c->v_l.push_back(v);
     }
     c->n_seq_max = c->p.n_seq_max > 0 ? c->p.n_seq_max : 8;
-    if (m->has_shift || m->bigram) c->seq_prev_tok.assign((size_t) c->n_seq_max, -1);
+    if (m->has_shift || m->bigram || m->has_seq_state) c->seq_prev_tok.assign((size_t) c->n_seq_max, -1);
+    if (m->has_seq_state) {
+        c->conv_state.assign((size_t) n_runs, nullptr);
+        c->tm_shift_state.assign((size_t) n_runs, nullptr);
+        c->rec_state.assign((size_t) n_runs, nullptr);
+        for (int run = 0; run < n_runs; ++run) {
+            const llm_layer_cfg & lc = m->lcfg[(size_t) m->runs[(size_t) run].il];
+            const int64_t S = c->n_seq_max;
+            int64_t conv_c = 0, rec = 0;
+            if (lc.mixer == LLM_MIX_MLSTM) rec = ggml_seq_state_size(2, lc.n_head, lc.dk, lc.dv);
+            else if (lc.mixer == LLM_MIX_DELTA) { conv_c = 2 * (int64_t) lc.n_head_kv * lc.dk + (int64_t) lc.n_head * lc.dv; rec = ggml_seq_state_size(1, lc.n_head, lc.dk, lc.dv); }
+            else if (lc.mixer == LLM_MIX_SIGMOID_WKV) {
+                conv_c = (int64_t) (lc.n_head + lc.n_head_kv) * lc.dk + (int64_t) lc.n_head_kv * lc.dv;
+                rec = ggml_seq_state_size(0, lc.tm_heads, lc.tm_dim, lc.tm_dim);
+                c->tm_shift_state[(size_t) run] = named(ggml_new_tensor_2d(c->ctx_kv, GGML_TYPE_F32, hp.n_embd, S), "time_mix_shift_state", run);
+            }
+            if (conv_c > 0 && lc.conv_taps > 1) c->conv_state[(size_t) run] = named(ggml_new_tensor_2d(c->ctx_kv, GGML_TYPE_F32, conv_c * (lc.conv_taps - 1), S), "conv_state", run);
+            if (rec > 0) c->rec_state[(size_t) run] = named(ggml_new_tensor_2d(c->ctx_kv, GGML_TYPE_F32, rec, S), "recurrence_state", run);
+        }
+    }
     if (m->has_shift) c->shift_state = named(ggml_new_tensor_3d(c->ctx_kv, GGML_TYPE_F32, hp.n_embd, c->n_seq_max + 1, n_runs), "shift_state", -1);
     c->buf_kv = ggml_backend_alloc_ctx_tensors_from_buft(c->ctx_kv, c->buft);
     if (!c->buf_kv) {
@@ -1875,7 +2341,8 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
     c->used_max = 0;
     c->galloc = ggml_gallocr_new(c->buft);
     // reserve the worst-case graph (full micro-batch over the full cache) so later graphs re-use one buffer
-    build_graph(c, std::min(c->p.n_ubatch, c->p.n_ctx), c->p.n_ctx, std::min(c->p.n_ubatch, c->p.n_ctx), m->has_shift ? std::min(c->n_seq_max, std::min(c->p.n_ubatch, c->p.n_ctx)) : 0);
+    build_graph(c, std::min(c->p.n_ubatch, c->p.n_ctx), c->p.n_ctx, std::min(c->p.n_ubatch, c->p.n_ctx),
+                (m->has_shift || m->has_seq_state) ? std::min(c->n_seq_max, std::min(c->p.n_ubatch, c->p.n_ctx)) : 0);
     if (!ggml_gallocr_reserve(c->galloc, c->gf)) {
         fprintf(stderr, "llm_context_new: failed to reserve the compute buffer\n");
         llm_context_free(c);
@@ -1889,6 +2356,7 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
             const size_t n_tok_pad = (nub + 63) / 64 * 64;
             size_t in_bytes = nub * (4 + 4 + 8 + 4) + std::max<size_t>(1, m->mask_rules.size()) * (n_tok_pad * (size_t) c->p.n_ctx * 4 + 64) + 256;
             in_bytes += nub * (4 + 4) + (size_t) c->n_seq_max * (4 + 8) + 4 * 64;  // bigram rows, token-shift sources, the sequences' last rows and state rows
+            in_bytes += (nub + (size_t) c->n_seq_max) * (size_t) (m->hist_rows + 4) * 4 + 4 * 64;  // predecessors, new state rows, rows grouped by sequence, the sequences' entries
             if (!c->p.flash_attn) in_bytes += nub * (size_t) n_embd_k * 8;
             in_bytes = (in_bytes + 255) / 256 * 256;
             c->pin_out_rows = 64;
@@ -2239,7 +2707,38 @@ static int decode_ubatch(llm_context * c, int n_tokens, const int32_t * tokens, 
                 new_prev_tok[(size_t) sq] = tokens[last_in_batch[(size_t) sq]];
             }
     }
-    const int n_seqs = m->has_shift ? (int) shift_last.size() : 0;
+    // layers with convolution / recurrence state: the batch rows of every sequence in their order, and from them where each token's predecessors are found (hist),
+    // where the state rows after the batch come from (upd), and the sequences' entries (info)
+    std::vector<int32_t> seq_hist, seq_upd, seq_tok, seq_info;
+    if (m->has_seq_state) {
+        const int S = c->n_seq_max, hs = m->hist_rows;
+        std::vector<std::vector<int>> rows((size_t) S);
+        for (int i = 0; i < n_tokens; ++i) rows[(size_t) (seq_id ? seq_id[i] : 0)].push_back(i);
+        seq_hist.assign((size_t) hs * n_tokens, -1);
+        for (int sq = 0; sq < S; ++sq) {
+            const std::vector<int> & r = rows[(size_t) sq];
+            if (r.empty()) continue;
+            const int n = (int) r.size();
+            for (int k = 0; k < n; ++k)
+                for (int d = 1; d <= hs; ++d) {
+                    int32_t code = -1;  // before the sequence's start
+                    if (pos[r[(size_t) k]] - d >= 0) code = d <= k ? r[(size_t) (k - d)] : -2 - (sq * 64 + (d - 1 - k));
+                    seq_hist[(size_t) r[(size_t) k] * hs + (d - 1)] = code;
+                }
+            const int last_pos = pos[r[(size_t) (n - 1)]];
+            for (int a = 0; a < hs; ++a) {
+                int32_t code = -1;
+                if (last_pos - a >= 0) code = a < n ? r[(size_t) (n - 1 - a)] : -2 - (sq * 64 + (a - n));
+                seq_upd.push_back(code);
+            }
+            seq_info.push_back((int32_t) seq_tok.size());
+            seq_info.push_back(n);
+            seq_info.push_back(sq);
+            seq_info.push_back(pos[r[0]] == 0 ? 1 : 0);
+            for (int k = 0; k < n; ++k) seq_tok.push_back(r[(size_t) k]);
+        }
+    }
+    const int n_seqs = m->has_shift ? (int) shift_last.size() : m->has_seq_state ? (int) (seq_info.size() / 4) : 0;
     graph_key key{n_tokens, n_kv, n_out_graph, n_seqs};
     bool rebuilt = false;
     if (!(c->p.graph_reuse && key == c->key && c->gf)) {
@@ -2279,10 +2778,18 @@ static int decode_ubatch(llm_context * c, int n_tokens, const int32_t * tokens, 
     };
     upload(c->inp_tokens, (size_t) n_tokens * 4, [&](char * d) { memcpy(d, tokens, (size_t) n_tokens * 4); });
     if (c->inp_pos) upload(c->inp_pos, (size_t) n_tokens * 4, [&](char * d) { memcpy(d, pos, (size_t) n_tokens * 4); });
-    upload(c->inp_k_idxs, (size_t) n_tokens * 8, [&](char * d) {
+    if (c->inp_k_idxs) upload(c->inp_k_idxs, (size_t) n_tokens * 8, [&](char * d) {
         int64_t * k = (int64_t *) d;
         for (int i = 0; i < n_tokens; ++i) k[i] = slots[i];
     });
+    if (c->inp_seq_hist) {
+        upload(c->inp_seq_hist, seq_hist.size() * 4, [&](char * d) { memcpy(d, seq_hist.data(), seq_hist.size() * 4); });
+        upload(c->inp_seq_upd, seq_upd.size() * 4, [&](char * d) { memcpy(d, seq_upd.data(), seq_upd.size() * 4); });
+    }
+    if (c->inp_seq_tok) {
+        upload(c->inp_seq_tok, seq_tok.size() * 4, [&](char * d) { memcpy(d, seq_tok.data(), seq_tok.size() * 4); });
+        upload(c->inp_seq_info, seq_info.size() * 4, [&](char * d) { memcpy(d, seq_info.data(), seq_info.size() * 4); });
+    }
     if (c->inp_v_idxs) {
         const int64_t n_embd_k = (int64_t) m->n_head_kv_l * hp.n_embd_head;
         upload(c->inp_v_idxs, (size_t) n_tokens * n_embd_k * 8, [&](char * d) {
@@ -2298,7 +2805,7 @@ static int decode_ubatch(llm_context * c, int n_tokens, const int32_t * tokens, 
         upload(c->inp_shift_last, (size_t) n_seqs * 4, [&](char * d) { memcpy(d, shift_last.data(), (size_t) n_seqs * 4); });
         upload(c->inp_shift_slot, (size_t) n_seqs * 8, [&](char * d) { memcpy(d, shift_slot.data(), (size_t) n_seqs * 8); });
     }
-    {
+    if (c->inp_mask) {
         // rows beyond n_tokens are padding (GGML_KQ_MASK_PAD) that no kernel reads: they are written once when the
         // graph is (re)built and skipped on re-use, which keeps the per-step upload at n_tokens * n_kv entries
         const int64_t n_tok_pad = c->inp_mask->ne[1];

@@ -61,7 +61,9 @@ struct llm_model * llm_model_load(const char * path, ggml_backend_buffer_type_t 
 /* A checkpoint FOLDER: config.json + model.safetensors.  config.json's "architecture" chooses the model class; today "Nigozen": a decoder whose
  * layers are listed one by one in the config (grouped-query attention with partial interleaved rotary positions, attention confined to chunks of
  * positions, a soft-max with a zero-score sink, value mixing with the first such layer, a sigmoid output gate, layer norms before and after every
- * sublayer, a dense erf-GELU or a top-k mixture-of-experts feed-forward, tied output matrix).  wtype: GGML_TYPE_BF16 keeps the matrices as stored
+ * sublayer, a dense erf-GELU or a top-k mixture-of-experts feed-forward, tied output matrix); "Zigipel" (latent and windowed attention, token shift, a
+ * repeated range of layers); "Rarelorn" (mixers with state per sequence: a matrix memory with exponential gates, a gated delta rule behind short
+ * convolutions, windowed sigmoid attention beside RWKV-style time mixing; experts chosen from a soft-max over all of them within the best groups).  wtype: GGML_TYPE_BF16 keeps the matrices as stored
  * (bf16 products, f32 accumulation); GGML_TYPE_F32 widens them at load (everything in 32-bit).  Norm weights and routers are always f32. */
 struct llm_model * llm_model_load_dir(const char * dir, ggml_backend_buffer_type_t buft, int wtype);
 /* the same model classes from the TEXT of a config.json and seeded random weights (benchmarks at sizes no file exists for) */
