@@ -139,13 +139,13 @@ NIGOZEN_SIZES = {
 }
 
 
-def nigozen_config(z, dense_only=False):
-    """layers alternate a dense and a mixture-of-experts feed-forward (dense_only: every layer dense); every layer mixes values and is confined to chunks"""
+def nigozen_config(z, dense_only=False, moe_only=False):
+    """layers alternate a dense and a mixture-of-experts feed-forward (dense_only: every layer dense; moe_only: every layer experts); every layer mixes values and is confined to chunks"""
     layers = []
     for il in range(z["layers"]):
         mixer = {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["hd"], "vdim": z["hd"], "mask": {"size": z["chunk"]}, "rot": {"base": 1e6, "dims": z["rot"]},
                  "scale": z["hd"] ** -0.5, "v_mix": True}
-        mlp = {"kind": "dense", "ff": z["ff"]} if (il % 2 == 0 or dense_only) else {"kind": "moe", "expert": {"ff": z["eff"]}, "router": {"experts": z["experts"], "top": z["top"]}}
+        mlp = {"kind": "dense", "ff": z["ff"]} if ((il % 2 == 0 and not moe_only) or dense_only) else {"kind": "moe", "expert": {"ff": z["eff"]}, "router": {"experts": z["experts"], "top": z["top"]}}
         layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
     return {"architecture": "Nigozen", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-5}, "vocab": z["vocab"], "width": z["width"]}
 
@@ -175,6 +175,27 @@ def zigipel_config(z):
             "loop": {"start": 1, "stop": 3, "times": 2}, "norm": {"eps": 1e-5}, "logit_scale": 0.5, "vocab": z["vocab"], "width": z["width"]}
 
 
+# ------------------------------------------------------------------------------------------------ --rarelorn: the class with state per sequence, beside Nigozen
+RARELORN_SIZES = {
+    # width, heads, key heads, head size (keys and values), window, taps, experts, top, expert ff (gated: three matrices), vocab.  Four layers (matrix memory, delta rule,
+    # sigmoid attention beside time mixing, delta rule), the middle two run twice: six layer runs, as many as the Nigozen model beside it has layers
+    "s": dict(width=1024, heads=8, kv=2, hd=64, window=512, taps=4, experts=8, top=2, eff=1024, vocab=32000),
+    "m": dict(width=2048, heads=16, kv=4, hd=128, window=1024, taps=4, experts=8, top=2, eff=2048, vocab=32000),
+    "l": dict(width=4096, heads=32, kv=8, hd=128, window=2048, taps=4, experts=8, top=2, eff=4096, vocab=32000),
+}
+
+
+def rarelorn_config(z):
+    mlp = {"kind": "moe", "expert": {"ff": z["eff"]}, "router": {"experts": z["experts"], "top": z["top"], "scale": 1.5, "groups": {"count": 4, "keep": 2}}}
+    H, G, D = z["heads"], z["kv"], z["hd"]
+    mlstm = {"type": "mlstm", "mlp": mlp, "mixer": {"heads": H, "dim": D, "vdim": D, "gate_cap": 15.0}}
+    delta = {"type": "delta", "mlp": mlp, "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": z["taps"]}}
+    par = {"type": "parallel", "mlp": mlp, "mixer": {"left_scale": 1.0, "right_scale": 1.0, "right": {"heads": z["width"] // 64, "dim": 64, "rank": 64},
+                                                       "left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": z["taps"], "mask": {"size": z["window"]}, "scale": D ** -0.5,
+                                                                "softcap": 50.0, "rot": {"base": 1e6, "dims": D // 2}}}}
+    return {"architecture": "Rarelorn", "layers": [mlstm, delta, par, delta], "loop": {"start": 1, "stop": 3, "times": 2}, "norm": {"eps": 1e-5}, "vocab": z["vocab"], "width": z["width"]}
+
+
 def bench_nigozen(args):
     """Prefill and decode throughput of Nigozen models (bf16 matrices, bf16 cache, random weights) at sizes that resemble real layers, beside the
     closest existing class at equal size: llama with f16 matrices and an f16 cache (same width, layers, heads, head size, dense ff and vocabulary;
@@ -190,7 +211,7 @@ def bench_nigozen(args):
 
     be = L.Backend(0)
     n_prompt, n_dec, ub = args.prefill, max(8, min(args.steps, 64)), args.ubatch
-    if args.zigipel and n_prompt == 2048:
+    if (args.zigipel or args.rarelorn) and n_prompt == 2048:
         # decoded positions 1984 .. 2047: a model confined to chunks of 512 / 1024 / 2048 positions then sees 449 .. 512 / 961 .. 1024 / 1985 .. 2048 cells, about as many as a
         # sliding window of the same length does (right behind a chunk's start it would see next to nothing, and the two decode steps would not compare)
         n_prompt = 1984
@@ -203,7 +224,7 @@ def bench_nigozen(args):
         prompt = rng.integers(0, n_vocab, n_prompt).tolist()
         res = {}
         best_p, best_d = None, None
-        for rep in range(2 if not args.zigipel else 4):  # the first pass warms up (graph capture, scratch growth); the Zigipel comparison keeps the best of the three that follow
+        for rep in range(2 if not (args.zigipel or args.rarelorn) else 4):  # the first pass warms up (graph capture, scratch growth); the Zigipel comparison keeps the best of the three that follow
             ctx.clear()
             be.synchronize()
             t0 = time.perf_counter()
@@ -215,8 +236,8 @@ def bench_nigozen(args):
                 assert rc == 0
             t2 = time.perf_counter()
             if rep > 0:
-                best_p = (t1 - t0) if best_p is None or not args.zigipel else min(best_p, t1 - t0)
-                best_d = (t2 - t1) if best_d is None or not args.zigipel else min(best_d, t2 - t1)
+                best_p = (t1 - t0) if best_p is None or not (args.zigipel or args.rarelorn) else min(best_p, t1 - t0)
+                best_d = (t2 - t1) if best_d is None or not (args.zigipel or args.rarelorn) else min(best_d, t2 - t1)
         if True:
             res = {"prefill_tok_s": round(n_prompt / best_p, 1), "decode_tok_s": round(n_dec / best_d, 1), "prefill_ms": round(best_p * 1e3, 2), "decode_ms_per_tok": round(best_d * 1e3 / n_dec, 3)}
         if os.environ.get("BENCH_NIGOZEN_CLASSES", "1") == "0":  # (a run under a profiler: its own kernel trace replaces the event-bracketed pass)
@@ -238,6 +259,28 @@ def bench_nigozen(args):
         ctx.free()
         return res
 
+    if args.rarelorn:  # Rarelorn beside Nigozen (every layer experts) with as many layers as Rarelorn has layer runs, equal width, heads, head size, vocabulary and expert parameters
+        out["metric"] = "rarelorn_vs_nigozen_tokens_per_s"
+        out["dtype"] = "bf16 (both)"
+        be.close()
+        for name in args.rarelorn.split(","):
+            z = RARELORN_SIZES[name]
+            zn = dict(width=z["width"], layers=6, heads=z["heads"], kv=z["kv"], hd=z["hd"], rot=z["hd"] // 2, chunk=z["window"], ff=0, experts=z["experts"], top=z["top"],
+                      eff=z["eff"] * 3 // 2, vocab=z["vocab"])
+            res = {}
+            for side, cfg in (("rarelorn", rarelorn_config(z)), ("nigozen_moe", nigozen_config(zn, moe_only=True))):
+                be = L.Backend(0)
+                mdl = Model(config_json=_json.dumps(cfg), seed=7, buft=be.buft, wtype=L.BF16)
+                res[side] = run(mdl, z["vocab"])
+                res[side]["weight_bytes"] = int(L.host().llm_model_total_bytes(mdl.m))
+                res[side]["stream_bytes_per_token"] = mdl.stream_bytes()
+                mdl.free()
+                be.close()
+            out["sizes"][name] = {"config": z, "rarelorn": res["rarelorn"], "nigozen_moe": res["nigozen_moe"],
+                                  "prefill_ratio": round(res["rarelorn"]["prefill_tok_s"] / res["nigozen_moe"]["prefill_tok_s"], 3),
+                                  "decode_ratio": round(res["rarelorn"]["decode_tok_s"] / res["nigozen_moe"]["decode_tok_s"], 3)}
+        print(_json.dumps(out))
+        return
     if args.zigipel:  # Zigipel beside Nigozen (all layers dense) with as many layers as Zigipel has layer runs, equal width, heads, head size and vocabulary
         out["metric"] = "zigipel_vs_nigozen_tokens_per_s"
         out["dtype"] = "bf16 (both)"
@@ -284,6 +327,8 @@ def main():
                     "print one JSON line and exit; the default workload is not run")
     ap.add_argument("--zigipel", default="", help="comma-separated sizes (s, m, l): time prefill and decode of Zigipel models (latent + windowed attention, token shift, a repeated range) "
                     "beside Nigozen models of equal size, print one JSON line and exit; the default workload is not run")
+    ap.add_argument("--rarelorn", default="", help="comma-separated sizes (s, m, l): time prefill and decode of Rarelorn models (matrix memory, gated delta rule, sigmoid attention beside "
+                    "time mixing, grouped expert router, a repeated range) beside Nigozen models of equal size, print one JSON line and exit; the default workload is not run")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
@@ -312,7 +357,7 @@ def main():
     ap.add_argument("--pmc-traffic", type=int, default=1, help="1: re-run a short decode under rocprofv3 --pmc FETCH_SIZE (own pass) for roofline.traffic")
     args = ap.parse_args()
 
-    if args.nigozen or args.zigipel:
+    if args.nigozen or args.zigipel or args.rarelorn:
         bench_nigozen(args)
         return
 
