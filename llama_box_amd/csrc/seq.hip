@@ -174,6 +174,18 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
             f = f >= per_tok ? f - per_tok : f;
         }
     };
+    // the raw gates of a parked block become what the recurrence uses — (beta, decay) or the capped log gates — once per block, two lanes a token, instead of in
+    // every token's own chain of instructions (the same formulas on the same values)
+    auto finish_gates = [&](float * dstb) {
+        if (KIND != SEQ_WKV6 && lane < 2 * TB) {
+            float * gp = dstb + (lane >> 1) * per_tok + off_g + (lane & 1);
+            const float x = *gp;
+            float y;
+            if (KIND == SEQ_DELTA) y = (lane & 1) ? expf(-a_exp * seq_softplus(x + dt_b)) : 1.0f / (1.0f + expf(-x));
+            else y = (lane & 1) ? seq_log_sigmoid(A.cap * tanhf((x + bf) / A.cap)) : A.cap * tanhf((x + bi) / A.cap);
+            *gp = y;
+        }
+    };
     float pre[SEQ_NV];
     if (lane < SEQ_MAX_TB) {
         rows_of[0][lane] = lane < count ? A.tok[begin + lane] : 0;
@@ -182,6 +194,8 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
     __syncthreads();
     fetch(rows_of[0], min(TB, count), pre);
     park(blk[0], pre);
+    __syncthreads();
+    finish_gates(blk[0]);
     __syncthreads();
     for (int b0 = 0, b = 0; b0 < count; b0 += TB, ++b) {
         const int n_here = min(TB, count - b0), n_next = min(TB, count - b0 - TB);
@@ -216,9 +230,7 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
                 }
                 o = quad_sum((p0 + p1) + (p2 + p3));
             } else if (KIND == SEQ_DELTA) {
-                const float b_pre = lt[off_g], a_pre = lt[off_g + 1];
-                const float beta = 1.0f / (1.0f + expf(-b_pre));
-                const float gdec = expf(-a_exp * seq_softplus(a_pre + dt_b));
+                const float beta = lt[off_g], gdec = lt[off_g + 1];
                 float kn[R], qn[R];
                 float k2a = 0.0f, k2b = 0.0f, q2a = 0.0f, q2b = 0.0f;
 #pragma unroll
@@ -260,8 +272,7 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
                 }
                 o = quad_sum((p0 + p1) + (p2 + p3));
             } else {
-                const float i_raw = lt[off_g] + bi, f_raw = lt[off_g + 1] + bf;
-                const float ig = A.cap * tanhf(i_raw / A.cap), fg = seq_log_sigmoid(A.cap * tanhf(f_raw / A.cap));
+                const float ig = lt[off_g], fg = lt[off_g + 1];
                 const float m_new = fmaxf(fg + mrun, ig);
                 const float ea = expf(fg + mrun - m_new), eb = expf(ig - m_new);
                 mrun = m_new;
@@ -291,6 +302,8 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
         if (n_next > 0) {
             park(blk[(b + 1) & 1], pre);
             if (lane < TB) rows_of[b & 1][lane] = row_after;
+            __syncthreads();
+            finish_gates(blk[(b + 1) & 1]);
         }
         __syncthreads();
     }
