@@ -11,10 +11,10 @@
 //   k_seq_conv        short causal convolution per channel over a sequence's history (taps inputs, the last one the token's own), optionally followed by SiLU;
 //                     several weight sets over the same input give several outputs (a token shift h + (h_prev - h) mu is the 2-tap case with weights (mu, 1 - mu))
 //   k_seq_conv_store  the last taps - 1 inputs of every sequence of the batch become its state
-//   k_seq_wkv6        o_t = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T, w = exp(-exp(w_pre + w0)) per key channel
-//   k_seq_delta       gated delta rule: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q — unit-length q, k, sigmoid beta and the decay
+//   k_seq_recurrence<SEQ_WKV6>   o_t = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T, w = exp(-exp(w_pre + w0)) per key channel
+//   k_seq_recurrence<SEQ_DELTA>  gated delta rule: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q — unit-length q, k, sigmoid beta and the decay
 //                     g = exp(-exp(A_log) softplus(a + dt_bias)) computed here from the raw projections
-//   k_seq_mlstm       matrix memory with exponential gates under a running maximum m: m' = max(f + m, i); S <- e^(f + m - m') S + e^(i - m') k v^T; n likewise with k;
+//   k_seq_recurrence<SEQ_MLSTM>  matrix memory with exponential gates under a running maximum m: m' = max(f + m, i); S <- e^(f + m - m') S + e^(i - m') k v^T; n likewise with k;
 //                     o = S^T q / (max(|n . q|, e^(-m')) + 1e-6); log gates capped by cap tanh(. / cap), f through log-sigmoid
 // All arithmetic is f32; the state is f32.  The three recurrences share one thread layout: a wave per (sequence of the batch, head, 4 value columns); value column j
 // of the head's state matrix is held by SIXTEEN neighbouring lanes (a DPP row), each owning a sixteenth of the key rows (neighbours) in registers; dot products over the key
