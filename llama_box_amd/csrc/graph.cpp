@@ -135,6 +135,9 @@ static int rope_exact_freq(const ggml_tensor * n) {
 //                                          mode 1  src (x, upd [hs, n_seq] i32, info [4, n_seq] i32) -> the state (a view of it): the sequences' last taps - 1 inputs
 //   RWKV_WKV6, op_params (H): src (r, k, v, w_pre [D H, T], w0 [D H], u [D H], state, tok [T] i32, info) -> [D, H, T]
 //   GATED_LINEAR_ATTN, op_params (kind 1 delta rule / 2 matrix memory, H, G, tag, cap, q scale): src (q, k [DK G, T], v [DV H, T], gates [2 H, T], params [2 H], state, tok, info) -> [DV, H, T]
+//                      kind 3 (delta rule, one decay per key channel): gates = a_pre [DK H, T], params = A_log [H] then dt_bias [DK H], src[8] = b_pre [H, T];
+//                      kind 4 (state-space duality): q = C, k = B [N G, T], v = x, gates = dt_pre [H, T], params = A_log, dt_bias, D [3 H]
+//   SSM_CONV mode 0 may carry src[4]: a bias [C, M] added before the activation
 static constexpr int32_t MI_SEQ_OP_TAG = 0x5E9;
 static bool seq_op_ok(const ggml_tensor * op) {
     if (op->op_params[3] != MI_SEQ_OP_TAG || op->type != GGML_TYPE_F32) return false;
@@ -148,11 +151,12 @@ static bool seq_op_ok(const ggml_tensor * op) {
         if (mode == 1) return taps >= 2 && i32c(src[1]) && i32c(src[2]) && src[1]->ne[0] >= taps - 1 && src[2]->ne[0] == 4 && src[1]->ne[1] == src[2]->ne[1] && ggml_abi_is_contiguous(op);
         if (mode != 0 || !f32c(src[1]) || !ggml_abi_is_contiguous(op)) return false;
         if (src[1]->ne[0] != taps || src[1]->ne[1] != src[0]->ne[0] || op->ne[0] != src[0]->ne[0] || op->ne[1] != src[0]->ne[1] || op->ne[2] != src[1]->ne[2]) return false;
+        if (src[4] && (!f32c(src[4]) || ggml_abi_nelements(src[4]) != src[0]->ne[0] * src[1]->ne[2])) return false;
         return taps == 1 || (f32c(src[2]) && i32c(src[3]) && src[3]->ne[0] >= taps - 1 && src[3]->ne[1] == src[0]->ne[1]);
     }
     const bool wkv = op->op == GGML_OP_RWKV_WKV6;
     const int kind = wkv ? SEQ_WKV6 : op->op_params[0];
-    if (!wkv && kind != SEQ_DELTA && kind != SEQ_MLSTM) return false;
+    if (!wkv && kind != SEQ_DELTA && kind != SEQ_MLSTM && kind != SEQ_DELTA_CH && kind != SEQ_SSD) return false;
     const int H = wkv ? op->op_params[0] : op->op_params[1], G = wkv ? H : op->op_params[2];
     const ggml_tensor * state = src[wkv ? 6 : 5], * tok = src[wkv ? 7 : 6], * info = src[wkv ? 8 : 7];
     if (H < 1 || G < 1 || H % G || !f32rows(src[0]) || !f32rows(src[1]) || !f32rows(src[2]) || !f32rows(src[3]) || !f32c(src[4]) || !f32c(state) || !i32c(tok) || !i32c(info)) return false;
@@ -161,7 +165,10 @@ static bool seq_op_ok(const ggml_tensor * op) {
     if (src[0]->ne[0] % G || src[2]->ne[0] % H) return false;
     const int64_t DK = src[0]->ne[0] / G, DV = src[2]->ne[0] / H;
     if (!seq_recurrence_ok((int) DK, (int) DV) || src[1]->ne[0] != DK * G || src[1]->ne[1] != T || src[2]->ne[1] != T || src[3]->ne[1] != T) return false;
-    if (src[3]->ne[0] != (wkv ? DK * H : 2 * H) || ggml_abi_nelements(src[4]) != (wkv ? DK * H : 2 * H) || (wkv && ggml_abi_nelements(src[5]) != DK * H)) return false;
+    const int64_t n_gates = (wkv || kind == SEQ_DELTA_CH) ? DK * H : kind == SEQ_SSD ? H : 2 * H;
+    const int64_t n_par = wkv ? DK * H : kind == SEQ_DELTA_CH ? H + DK * H : kind == SEQ_SSD ? 3 * H : 2 * H;
+    if (src[3]->ne[0] != n_gates || ggml_abi_nelements(src[4]) != n_par || (wkv && ggml_abi_nelements(src[5]) != DK * H)) return false;
+    if (kind == SEQ_DELTA_CH && (!f32rows(src[8]) || src[8]->ne[0] != H || src[8]->ne[1] != T)) return false;
     if (ggml_abi_nelements(tok) != T || info->ne[0] != 4 || state->ne[0] != seq_recurrence_state_floats(kind, H, (int) DK, (int) DV)) return false;
     return op->ne[0] == DV && op->ne[1] == H && op->ne[2] == T && ggml_abi_is_contiguous(op);
 }
@@ -2078,10 +2085,10 @@ static int try_fuse_add_chain(exec_state & st, int i) {
     return 3;
 }
 
-// ROPE over a frequency table, rotate-half over the whole row: the shapes the two fusions below serve
+// ROPE over a frequency table, over the whole row, as rotate-half or as neighbouring pairs: the shapes the two fusions below serve
 static bool rope_table_plain(const ggml_tensor * n) {
     const ggml_tensor * a = n->src[0];
-    return n->op_params[3] == 2 && n->src[2] && (n->op_params[2] == GGML_ROPE_TYPE_NEOX) && n->op_params[1] == a->ne[0] && (a->ne[0] % 2) == 0 && a->type == GGML_TYPE_F32 && a->nb[0] == 4 &&
+    return n->op_params[3] == 2 && n->src[2] && (n->op_params[2] == GGML_ROPE_TYPE_NEOX || n->op_params[2] == 0) && n->op_params[1] == a->ne[0] && (a->ne[0] % 2) == 0 && a->type == GGML_TYPE_F32 && a->nb[0] == 4 &&
            n->type == GGML_TYPE_F32 && n->ne[3] == 1 && n->src[1]->type == GGML_TYPE_I32 && n->src[2]->type == GGML_TYPE_F32 && ggml_abi_is_contiguous(n->src[2]);
 }
 // ROPE(k_r; table) -> RESHAPE -> CONCAT(latent, .; dim 0) -> SET_ROWS(cache): the latent cache row written in place.  Returns the nodes consumed
@@ -2096,7 +2103,7 @@ static int try_fuse_latent_row_store(exec_state & st, int i) {
     if (lat->type != GGML_TYPE_F32 || lat->nb[0] != 4 || lat->ne[1] != T || lat->ne[2] != 1 || lat->ne[3] != 1 || idx->type != GGML_TYPE_I64 || !ggml_abi_is_contiguous(idx) || ggml_abi_nelements(idx) != T) return 0;
     if (!(sr->type == GGML_TYPE_F32 || sr->type == GGML_TYPE_BF16 || sr->type == GGML_TYPE_F16) || sr->nb[0] != ggml_abi_type_size(sr->type) || sr->ne[0] != lat->ne[0] + n->ne[0]) return 0;
     if (!single_use(st, n) || !single_use(st, rs) || !single_use(st, cc)) return 0;
-    launch_latent_row_store(st.c->stream, TD(lat), TD(n->src[0]), TD(n->src[1]), (const float *) n->src[2]->data, ggml_abi_op_param_f32(n, 8), (int) n->ne[0], (const int64_t *) idx->data, TD(sr));
+    launch_latent_row_store(st.c->stream, TD(lat), TD(n->src[0]), TD(n->src[1]), (const float *) n->src[2]->data, ggml_abi_op_param_f32(n, 8), (int) n->ne[0], n->op_params[2] == GGML_ROPE_TYPE_NEOX, (const int64_t *) idx->data, TD(sr));
     st.c->st.kernel_launches++;
     st.c->st.fused_nodes += 3;
     return 4;
@@ -2110,7 +2117,7 @@ static int try_fuse_concat_rope(exec_state & st, int i) {
     if (cc->op != GGML_OP_CONCAT || cc->op_params[0] != 0 || cc->src[1] != n || !single_use(st, n) || !is_f32_contig(cc)) return 0;
     const ggml_tensor * qa = cc->src[0];
     if (qa->type != GGML_TYPE_F32 || qa->nb[0] != 4 || qa->ne[1] != n->ne[1] || qa->ne[2] != n->ne[2] || qa->ne[3] != 1 || ranges_overlap(cc, qa) || ranges_overlap(cc, n->src[0])) return 0;
-    launch_concat_rope(st.c->stream, TD(qa), TD(n->src[0]), TD(n->src[1]), (const float *) n->src[2]->data, ggml_abi_op_param_f32(n, 8), TD(cc));
+    launch_concat_rope(st.c->stream, TD(qa), TD(n->src[0]), TD(n->src[1]), (const float *) n->src[2]->data, ggml_abi_op_param_f32(n, 8), n->op_params[2] == GGML_ROPE_TYPE_NEOX, TD(cc));
     st.c->st.kernel_launches++;
     st.c->st.fused_nodes += 1;
     return 2;
@@ -2477,7 +2484,8 @@ static int run_node(exec_state & st, int i) {
                 launch_seq_conv_store(s, TD(a), (float *) n->data, (const int32_t *) n->src[1]->data, (int) n->src[1]->ne[0], (const int32_t *) n->src[2]->data, (int) n->src[2]->ne[1], taps);
             } else {
                 timed_scope ts(c, "seq_conv", (double) ggml_abi_nbytes(a) + (double) ggml_abi_nbytes(n));
-                launch_seq_conv(s, TD(a), (const float *) n->src[1]->data, n->src[2] ? (const float *) n->src[2]->data : nullptr, n->src[3] ? (const int32_t *) n->src[3]->data : nullptr,
+                launch_seq_conv(s, TD(a), (const float *) n->src[1]->data, n->src[4] ? (const float *) n->src[4]->data : nullptr, n->src[2] ? (const float *) n->src[2]->data : nullptr,
+                                n->src[3] ? (const int32_t *) n->src[3]->data : nullptr,
                                 n->src[3] ? (int) n->src[3]->ne[0] : 0, TD(n), taps, n->op_params[1]);
             }
             c->st.kernel_launches++;
@@ -2489,6 +2497,7 @@ static int run_node(exec_state & st, int i) {
             const ggml_tensor * state = n->src[wkv ? 6 : 5], * tok = n->src[wkv ? 7 : 6], * info = n->src[wkv ? 8 : 7];
             seq_rec_args ra;
             ra.q = TD(n->src[0]); ra.k = TD(n->src[1]); ra.v = TD(n->src[2]); ra.g = TD(n->src[3]);
+            ra.b = TD(kind == SEQ_DELTA_CH ? n->src[8] : n->src[3]);
             ra.p0 = (const float *) n->src[4]->data;
             ra.p1 = wkv ? (const float *) n->src[5]->data : nullptr;
             ra.state = (float *) state->data;

@@ -259,8 +259,8 @@ void launch_copy_rows_indexed(hipStream_t s, const tdesc & a, const int32_t * sr
 void launch_geglu_bias(hipStream_t s, const float * g, const float * bg, const float * u, const float * bu, float * d, int64_t n, int64_t rows);
 void launch_add_chain(hipStream_t s, const float * x, const float * a, const float * y, const float * b, float * d, int64_t n, int64_t rows);
 void launch_mul_sigmoid_rows(hipStream_t s, const float * x, const float * g, float * d, int64_t n, int64_t rows);
-void launch_latent_row_store(hipStream_t s, const tdesc & lat, const tdesc & kr, const tdesc & pos, const float * freq, float mag, int n_rot, const int64_t * idx, const tdesc & cache);
-void launch_concat_rope(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & pos, const float * freq, float mag, const tdesc & d);
+void launch_latent_row_store(hipStream_t s, const tdesc & lat, const tdesc & kr, const tdesc & pos, const float * freq, float mag, int n_rot, bool neox, const int64_t * idx, const tdesc & cache);
+void launch_concat_rope(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & pos, const float * freq, float mag, bool neox, const tdesc & d);
 void launch_get_rows(hipStream_t s, const tdesc & src, const tdesc & idx, const tdesc & dst);
 void launch_set_rows(hipStream_t s, const tdesc & src, const tdesc & idx, const tdesc & dst);
 void launch_cpy_q8_0(hipStream_t s, const void * src, void * dst, int64_t n_values, bool to_q8);  // contiguous Q8_0 <-> F32 (K-shift of a quantised cache)
@@ -380,12 +380,14 @@ bool repack_q80_supported(int type, int64_t K, int64_t N, int64_t nb1);  // Q8_0
 void launch_repack_q80_panels(hipStream_t s, const void * src, void * dst, int64_t K, int64_t N, int64_t nb1);
 
 // ---- layers with state per sequence (seq.hip): short convolutions over a sequence's history and three recurrences over a matrix state per head
-void launch_seq_conv(hipStream_t s, const tdesc & x, const float * w, const float * state, const int32_t * hist, int hs, const tdesc & dst, int taps, int act);
+void launch_seq_conv(hipStream_t s, const tdesc & x, const float * w, const float * bias, const float * state, const int32_t * hist, int hs, const tdesc & dst, int taps, int act);
 void launch_seq_conv_store(hipStream_t s, const tdesc & x, float * state, const int32_t * upd, int hs, const int32_t * info, int n_seqs, int taps);
 struct seq_rec_args {
     tdesc q, k, v;             // [rows, T] f32 (rows contiguous): q / r, k and v of all heads
-    tdesc g;                   // wkv6: w_pre [D H, T]; delta: (b_pre, a_pre) [2 H, T]; mlstm: (i_pre, f_pre) [2 H, T]
-    const float * p0;          // wkv6: w0 [D H]; delta: A_log [H] then dt_bias [H]; mlstm: bias of (i, f) [2 H]
+    tdesc g;                   // wkv6: w_pre [D H, T]; delta: (b_pre, a_pre) [2 H, T]; mlstm: (i_pre, f_pre) [2 H, T]; channel decay: a_pre [DK H, T]; state space: dt_pre [H, T]
+    tdesc b;                   // channel decay: b_pre [H, T]
+    const float * p0;          // wkv6: w0 [D H]; delta: A_log [H] then dt_bias [H]; mlstm: bias of (i, f) [2 H]; channel decay: A_log [H] then dt_bias [DK H];
+                               // state space: A_log [H], dt_bias [H], D [H]
     const float * p1;          // wkv6: u [D H]
     float * state;             // per slot: H matrices of 4 ceil(DK / 4) DV values, then (mlstm) H x DK normaliser entries and H running maxima
     int64_t state_stride;      // floats per slot
@@ -396,7 +398,7 @@ struct seq_rec_args {
     float cap, qscale;
 };
 
-enum { SEQ_WKV6 = 0, SEQ_DELTA = 1, SEQ_MLSTM = 2 };
+enum { SEQ_WKV6 = 0, SEQ_DELTA = 1, SEQ_MLSTM = 2, SEQ_DELTA_CH = 3, SEQ_SSD = 4 };
 int64_t seq_recurrence_state_floats(int kind, int H, int DK, int DV);
 bool seq_recurrence_ok(int DK, int DV);
 void launch_seq_recurrence(hipStream_t s, int kind, const seq_rec_args & a, int n_seqs);

@@ -1314,9 +1314,9 @@ void launch_mul_sigmoid_rows(hipStream_t s, const float * x, const float * g, fl
     if (total == 0) return;
     hipLaunchKernelGGL(k_mul_sigmoid_rows, dim3((unsigned) std::min<int64_t>((total + 255) / 256, 4096)), dim3(256), 0, s, x, g, d, n, total);
 }
-// a latent cache row: [lat[t] (n_lat values) | rotate-half(kr[t]) (n_rot values, frequency table)] stored as row idx[t] of the cache in its type
-// (ROPE -> CONCAT dim 0 -> SET_ROWS)
-__global__ void __launch_bounds__(128) k_latent_row_store(const tdesc lat, const tdesc kr, const tdesc pos, const float * __restrict__ freq, const float mag, const int n_rot,
+// a latent cache row: [lat[t] (n_lat values) | rotated kr[t] (n_rot values, frequency table; pairs (i, i + n_rot / 2) when `neox`, else (2i, 2i + 1))] stored as row idx[t] of
+// the cache in its type (ROPE -> CONCAT dim 0 -> SET_ROWS)
+__global__ void __launch_bounds__(128) k_latent_row_store(const tdesc lat, const tdesc kr, const tdesc pos, const float * __restrict__ freq, const float mag, const int n_rot, const bool neox,
                                                           const int64_t * __restrict__ idx, char * __restrict__ cache, const int64_t cache_nb1, const int cache_type) {
     const int64_t t = blockIdx.x;
     const int64_t n_lat = lat.ne[0];
@@ -1329,17 +1329,18 @@ __global__ void __launch_bounds__(128) k_latent_row_store(const tdesc lat, const
     for (int ip = threadIdx.x; ip < half; ip += blockDim.x) {
         float cs, sn;
         rope_cos_sin_table(ip, pos_f, freq, mag, cs, sn);
-        const float x0 = r[ip], x1 = r[ip + half];
-        store_as(row, cache_type, n_lat + ip, x0 * cs - x1 * sn);
-        store_as(row, cache_type, n_lat + ip + half, x0 * sn + x1 * cs);
+        const int ia = neox ? ip : 2 * ip, ib = neox ? ip + half : 2 * ip + 1;
+        const float x0 = r[ia], x1 = r[ib];
+        store_as(row, cache_type, n_lat + ia, x0 * cs - x1 * sn);
+        store_as(row, cache_type, n_lat + ib, x0 * sn + x1 * cs);
     }
 }
-void launch_latent_row_store(hipStream_t s, const tdesc & lat, const tdesc & kr, const tdesc & pos, const float * freq, float mag, int n_rot, const int64_t * idx, const tdesc & cache) {
+void launch_latent_row_store(hipStream_t s, const tdesc & lat, const tdesc & kr, const tdesc & pos, const float * freq, float mag, int n_rot, bool neox, const int64_t * idx, const tdesc & cache) {
     if (lat.ne[1] == 0) return;
-    hipLaunchKernelGGL(k_latent_row_store, dim3((unsigned) lat.ne[1]), dim3(128), 0, s, lat, kr, pos, freq, mag, n_rot, idx, cache.data, cache.nb[1], cache.type);
+    hipLaunchKernelGGL(k_latent_row_store, dim3((unsigned) lat.ne[1]), dim3(128), 0, s, lat, kr, pos, freq, mag, n_rot, neox, idx, cache.data, cache.nb[1], cache.type);
 }
-// the query rows of latent attention: d[.., h, t] = [a[.., h, t] (n_a values, any strides) | rotate-half(b[.., h, t]) (n_rot values, frequency table)] (ROPE -> CONCAT dim 0)
-__global__ void __launch_bounds__(128) k_concat_rope(const tdesc a, const tdesc b, const tdesc pos, const float * __restrict__ freq, const float mag, const tdesc d) {
+// the query rows of latent attention: d[.., h, t] = [a[.., h, t] (n_a values, any strides) | rotated b[.., h, t] (n_rot values, frequency table, pairs as above)] (ROPE -> CONCAT dim 0)
+__global__ void __launch_bounds__(128) k_concat_rope(const tdesc a, const tdesc b, const tdesc pos, const float * __restrict__ freq, const float mag, const bool neox, const tdesc d) {
     const int64_t h = blockIdx.x, t = blockIdx.y;
     const int64_t n_a = a.ne[0];
     const int half = (int) (b.ne[0] / 2);
@@ -1351,14 +1352,15 @@ __global__ void __launch_bounds__(128) k_concat_rope(const tdesc a, const tdesc 
     for (int ip = threadIdx.x; ip < half; ip += blockDim.x) {
         float cs, sn;
         rope_cos_sin_table(ip, pos_f, freq, mag, cs, sn);
-        const float x0 = r[ip], x1 = r[ip + half];
-        out[n_a + ip] = x0 * cs - x1 * sn;
-        out[n_a + ip + half] = x0 * sn + x1 * cs;
+        const int ia = neox ? ip : 2 * ip, ib = neox ? ip + half : 2 * ip + 1;
+        const float x0 = r[ia], x1 = r[ib];
+        out[n_a + ia] = x0 * cs - x1 * sn;
+        out[n_a + ib] = x0 * sn + x1 * cs;
     }
 }
-void launch_concat_rope(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & pos, const float * freq, float mag, const tdesc & d) {
+void launch_concat_rope(hipStream_t s, const tdesc & a, const tdesc & b, const tdesc & pos, const float * freq, float mag, bool neox, const tdesc & d) {
     if (d.ne[1] * d.ne[2] == 0) return;
-    hipLaunchKernelGGL(k_concat_rope, dim3((unsigned) d.ne[1], (unsigned) d.ne[2]), dim3(128), 0, s, a, b, pos, freq, mag, d);
+    hipLaunchKernelGGL(k_concat_rope, dim3((unsigned) d.ne[1], (unsigned) d.ne[2]), dim3(128), 0, s, a, b, pos, freq, mag, neox, d);
 }
 
 // a x + b y (k_axpby's arithmetic) stored as rows of a cache: row t of n values goes to cache row idx[t]

@@ -14,6 +14,10 @@
 //   k_seq_recurrence<SEQ_WKV6>   o_t = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T, w = exp(-exp(w_pre + w0)) per key channel
 //   k_seq_recurrence<SEQ_DELTA>  gated delta rule: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q — unit-length q, k, sigmoid beta and the decay
 //                     g = exp(-exp(A_log) softplus(a + dt_bias)) computed here from the raw projections
+//   k_seq_recurrence<SEQ_DELTA_CH>  the delta rule with ONE DECAY PER KEY CHANNEL: S <- diag(g) S with g = exp(-exp(A_log) softplus(a + dt_bias)) per (head, key row), the
+//                     raw a [DK H, T] being a projection of its own; beta = sigmoid(b_pre) from a [H, T] projection; the rest as SEQ_DELTA
+//   k_seq_recurrence<SEQ_SSD>    state-space duality (Mamba-2): dt = softplus(dt_pre + dt_bias); S <- exp(-exp(A_log) dt) S + dt B x^T; y = S^T C + D x, with B as the keys,
+//                     C as the queries (grouped: head h reads group h / (H / G)) and x as the values
 //   k_seq_recurrence<SEQ_MLSTM>  matrix memory with exponential gates under a running maximum m: m' = max(f + m, i); S <- e^(f + m - m') S + e^(i - m') k v^T; n likewise with k;
 //                     o = S^T q / (max(|n . q|, e^(-m')) + 1e-6); log gates capped by cap tanh(. / cap), f through log-sigmoid
 // All arithmetic is f32; the state is f32.  The three recurrences share one thread layout: a wave per (sequence of the batch, head, 4 value columns); value column j
@@ -41,9 +45,9 @@ __device__ __forceinline__ float seq_hist_value(const int code, const int c, con
 
 __device__ __forceinline__ float seq_silu(const float z) { return z / (1.0f + expf(-z)); }
 
-// y[c, t, m] = act(sum_j w[j, c, m] * x_(t - (taps - 1 - j))[c])
-__global__ void __launch_bounds__(256) k_seq_conv(const tdesc x, const float * __restrict__ w, const float * __restrict__ state, const int32_t * __restrict__ hist, const int hs,
-                                                  const tdesc dst, const int taps, const int act) {
+// y[c, t, m] = act(sum_j w[j, c, m] * x_(t - (taps - 1 - j))[c] + bias[c, m])   (bias may be null)
+__global__ void __launch_bounds__(256) k_seq_conv(const tdesc x, const float * __restrict__ w, const float * __restrict__ bias, const float * __restrict__ state,
+                                                  const int32_t * __restrict__ hist, const int hs, const tdesc dst, const int taps, const int act) {
     const int64_t C = x.ne[0], t = blockIdx.y;
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
@@ -57,6 +61,7 @@ __global__ void __launch_bounds__(256) k_seq_conv(const tdesc x, const float * _
 #pragma unroll
         for (int d = SEQ_MAX_TAPS - 1; d >= 0; --d)
             if (d < taps) y = fmaf(wc[taps - 1 - d], xv[d], y);  // oldest input first
+        if (bias) y += bias[m * C + c];
         ((float *) (dst.data + t * dst.nb[1] + m * dst.nb[2]))[c] = act ? seq_silu(y) : y;
     }
 }
@@ -75,9 +80,9 @@ __global__ void __launch_bounds__(256) k_seq_conv_store(const tdesc x, float * _
         if (a < taps - 1) state[((int64_t) slot * (taps - 1) + a) * C + c] = nv[a];  // (every value was read before the first is written: the rows shift in place)
 }
 
-void launch_seq_conv(hipStream_t s, const tdesc & x, const float * w, const float * state, const int32_t * hist, int hs, const tdesc & dst, int taps, int act) {
+void launch_seq_conv(hipStream_t s, const tdesc & x, const float * w, const float * bias, const float * state, const int32_t * hist, int hs, const tdesc & dst, int taps, int act) {
     if (x.ne[1] == 0 || x.ne[0] == 0) return;
-    hipLaunchKernelGGL(k_seq_conv, dim3((unsigned) ((x.ne[0] + 255) / 256), (unsigned) x.ne[1]), dim3(256), 0, s, x, w, state, hist, hs, dst, taps, act);
+    hipLaunchKernelGGL(k_seq_conv, dim3((unsigned) ((x.ne[0] + 255) / 256), (unsigned) x.ne[1]), dim3(256), 0, s, x, w, bias, state, hist, hs, dst, taps, act);
 }
 void launch_seq_conv_store(hipStream_t s, const tdesc & x, float * state, const int32_t * upd, int hs, const int32_t * info, int n_seqs, int taps) {
     if (n_seqs == 0 || x.ne[0] == 0 || taps < 2) return;
@@ -99,7 +104,7 @@ __device__ __forceinline__ float seq_log_sigmoid(const float z) { return fminf(z
 // One WAVE per (sequence of the batch, head, group of 4 value columns).  The tokens' vectors come in blocks of TB tokens: while block b is worked on out of LDS, block
 // b + 1 travels from memory into registers (one trip to memory per block, not per token) and is written to the other LDS buffer at the end; the batch rows of block b + 2
 // are fetched at the same time, so that no load ever waits for an address that is itself on its way.  A token's entries in a block: k [DK], q [DK], (wkv6: decay [DK]),
-// the wave's 4 values, (delta / matrix memory: the head's two raw gates).
+// the wave's 4 values, (delta / state space / matrix memory: the head's raw gates).
 constexpr int SEQ_COLS = 4;        // value columns of a wave
 constexpr int SEQ_LPC = 16;        // lanes per value column: each owns a sixteenth of the key rows
 constexpr int SEQ_NV = 32;         // registers a lane lends to the block on its way
@@ -107,6 +112,14 @@ constexpr int SEQ_MAX_TB = 16;     // tokens of a block at most
 
 // key rows a lane owns: a sixteenth of the head's rows, rounded up to whole groups of four (its rows are neighbours, read from LDS sixteen bytes at a time)
 static inline __host__ __device__ int seq_rows_per_lane(const int DK) { return (((DK + SEQ_LPC - 1) / SEQ_LPC) + 3) / 4 * 4; }
+// which kinds carry a decay per key channel among a token's entries, and which carry raw gates of the head
+static inline __host__ __device__ bool seq_has_w(const int kind) { return kind == SEQ_WKV6 || kind == SEQ_DELTA_CH; }
+static inline __host__ __device__ bool seq_has_gates(const int kind) { return kind != SEQ_WKV6; }
+// floats a token occupies in a staged block (at least a wave's stride: the walk over a block's entries then crosses at most one token per step)
+static inline __host__ __device__ int seq_per_tok(const int kind, const int DK) {
+    const int n = (seq_has_w(kind) ? 3 : 2) * SEQ_LPC * seq_rows_per_lane(DK) + SEQ_COLS + (seq_has_gates(kind) ? 4 : 0);
+    return n > 64 ? n : 64;
+}
 
 template <int KIND, int R, bool EXACT>   // R: key rows per lane at most (a multiple of 4); EXACT: exactly R (no test around a group of four rows)
 __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, const int TB) {
@@ -119,8 +132,9 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
     const bool col = j < DV;
     const int RL = seq_rows_per_lane(DK), KP = SEQ_LPC * RL;  // lane ks owns rows ks RL .. ks RL + RL - 1; a token's key-sized vectors are padded with zeros to KP entries
     const int kh = KIND == SEQ_WKV6 ? h : h / (H / A.G);
-    const int off_w = 2 * KP, off_v = KIND == SEQ_WKV6 ? 3 * KP : 2 * KP, off_g = off_v + SEQ_COLS;
-    const int per_tok = max(64, off_g + (KIND == SEQ_WKV6 ? 0 : 4));  // (at least a wave's stride: the walk over a block's entries then crosses at most one token per step)
+    constexpr bool HAS_W = KIND == SEQ_WKV6 || KIND == SEQ_DELTA_CH, HAS_G = KIND != SEQ_WKV6, IS_DELTA = KIND == SEQ_DELTA || KIND == SEQ_DELTA_CH;
+    const int off_w = 2 * KP, off_v = HAS_W ? 3 * KP : 2 * KP, off_g = off_v + SEQ_COLS;
+    const int per_tok = seq_per_tok(KIND, DK);
     float * __restrict__ Sm = A.state + (int64_t) slot * A.state_stride + (int64_t) h * RL * DV * SEQ_LPC;
     float * __restrict__ Nm = A.state + (int64_t) slot * A.state_stride + (int64_t) H * RL * DV * SEQ_LPC + (int64_t) h * DK;
     float * __restrict__ Mm = A.state + (int64_t) slot * A.state_stride + (int64_t) H * RL * DV * SEQ_LPC + (int64_t) H * DK + h;
@@ -136,8 +150,9 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
         if (KIND == SEQ_WKV6) { const float uv = A.p1[h * DK + (ok ? i : 0)]; uu[ii] = ok ? uv : 0.0f; } else uu[ii] = 0.0f;
     }
     float mrun = (KIND == SEQ_MLSTM && !reset) ? *Mm : 0.0f;
-    const float a_exp = KIND == SEQ_DELTA ? expf(A.p0[h]) : 0.0f;
-    const float dt_b = KIND == SEQ_DELTA ? A.p0[H + h] : 0.0f;
+    const float a_exp = (IS_DELTA || KIND == SEQ_SSD) ? expf(A.p0[h]) : 0.0f;
+    const float dt_b = (KIND == SEQ_DELTA || KIND == SEQ_SSD) ? A.p0[H + h] : 0.0f;
+    const float d_skip = KIND == SEQ_SSD ? A.p0[2 * H + h] : 0.0f;
     const float bi = KIND == SEQ_MLSTM ? A.p0[h] : 0.0f, bf = KIND == SEQ_MLSTM ? A.p0[H + h] : 0.0f;
 
     // entry e = lane + 64 i of a block (token u = e / per_tok, field f = e % per_tok) read from memory; `rows`: the block's batch rows
@@ -146,16 +161,18 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
 #pragma unroll
         for (int i = 0; i < SEQ_NV; ++i) {
             // which tensor, which entry: selected without branches, an entry that does not exist reads entry 0 of the block's first token (32 loads in flight together)
-            const bool is_k = f < KP, is_q = !is_k && f < 2 * KP, is_w = KIND == SEQ_WKV6 && !is_k && !is_q && f < off_v, is_v = !is_k && !is_q && !is_w && f < off_g;
+            const bool is_k = f < KP, is_q = !is_k && f < 2 * KP, is_w = HAS_W && !is_k && !is_q && f < off_v, is_v = !is_k && !is_q && !is_w && f < off_g;
             const int fe = is_k ? f : is_q ? f - KP : is_w ? f - off_w : is_v ? f - off_v : f - off_g;
-            const bool valid = u < n_tok && (is_v ? j0 + fe < DV : (is_k || is_q || is_w) ? fe < DK : (KIND != SEQ_WKV6 && fe < 2));
-            const char * base = is_k ? A.k.data : is_q ? A.q.data : is_v ? A.v.data : A.g.data;
-            const int64_t nb1 = is_k ? A.k.nb[1] : is_q ? A.q.nb[1] : is_v ? A.v.nb[1] : A.g.nb[1];
-            const int idx = (is_k || is_q) ? kh * DK + fe : is_w ? h * DK + fe : is_v ? h * DV + j0 + fe : fe * H + h;
+            // gates of the head: two raw projections (delta: b, a; matrix memory: i, f), one of its own tensor (channel decay: b), or one read twice (state space: dt)
+            const bool valid = u < n_tok && (is_v ? j0 + fe < DV : (is_k || is_q || is_w) ? fe < DK : (HAS_G && fe < (KIND == SEQ_DELTA_CH ? 1 : 2)));
+            const bool is_gate = !is_k && !is_q && !is_w && !is_v;
+            const char * base = is_k ? A.k.data : is_q ? A.q.data : is_v ? A.v.data : (KIND == SEQ_DELTA_CH && is_gate) ? A.b.data : A.g.data;
+            const int64_t nb1 = is_k ? A.k.nb[1] : is_q ? A.q.nb[1] : is_v ? A.v.nb[1] : (KIND == SEQ_DELTA_CH && is_gate) ? A.b.nb[1] : A.g.nb[1];
+            const int idx = (is_k || is_q) ? kh * DK + fe : is_w ? h * DK + fe : is_v ? h * DV + j0 + fe : (KIND == SEQ_DELTA_CH || KIND == SEQ_SSD) ? h : fe * H + h;
             const int64_t t = rows[valid ? u : 0];
             float val = ((const float *) (base + t * nb1))[valid ? idx : 0];
-            if (KIND == SEQ_WKV6) {
-                const float off = A.p0[(is_w && valid) ? h * DK + fe : 0];
+            if (HAS_W) {  // the decay's offset: w0 (time mixing), or the dt_bias entries behind the heads' A_log (channel decay)
+                const float off = A.p0[(is_w && valid) ? (KIND == SEQ_DELTA_CH ? H : 0) + h * DK + fe : 0];
                 val = is_w ? val + off : val;
             }
             pre[i] = valid ? val : 0.0f;
@@ -169,7 +186,8 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
         int f = lane >= per_tok ? lane - per_tok : lane;
 #pragma unroll
         for (int i = 0; i < SEQ_NV; ++i) {
-            if (lane + 64 * i < TB * per_tok) dstb[lane + 64 * i] = (KIND == SEQ_WKV6 && f >= off_w && f < off_v) ? expf(-expf(pre[i])) : pre[i];
+            if (lane + 64 * i < TB * per_tok)
+                dstb[lane + 64 * i] = (HAS_W && f >= off_w && f < off_v) ? (KIND == SEQ_WKV6 ? expf(-expf(pre[i])) : expf(-a_exp * seq_softplus(pre[i]))) : pre[i];
             f += 64;
             f = f >= per_tok ? f - per_tok : f;
         }
@@ -177,11 +195,13 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
     // the raw gates of a parked block become what the recurrence uses — (beta, decay) or the capped log gates — once per block, two lanes a token, instead of in
     // every token's own chain of instructions (the same formulas on the same values)
     auto finish_gates = [&](float * dstb) {
-        if (KIND != SEQ_WKV6 && lane < 2 * TB) {
+        if (HAS_G && lane < 2 * TB) {
             float * gp = dstb + (lane >> 1) * per_tok + off_g + (lane & 1);
             const float x = *gp;
             float y;
             if (KIND == SEQ_DELTA) y = (lane & 1) ? expf(-a_exp * seq_softplus(x + dt_b)) : 1.0f / (1.0f + expf(-x));
+            else if (KIND == SEQ_DELTA_CH) y = (lane & 1) ? x : 1.0f / (1.0f + expf(-x));
+            else if (KIND == SEQ_SSD) { const float dt = seq_softplus(x + dt_b); y = (lane & 1) ? expf(-a_exp * dt) : dt; }  // (step size, decay)
             else y = (lane & 1) ? seq_log_sigmoid(A.cap * tanhf((x + bf) / A.cap)) : A.cap * tanhf((x + bi) / A.cap);
             *gp = y;
         }
@@ -229,7 +249,25 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
                     }
                 }
                 o = quad_sum((p0 + p1) + (p2 + p3));
-            } else if (KIND == SEQ_DELTA) {
+            } else if (KIND == SEQ_SSD) {
+                const float dtv = lt[off_g] * vj, dec = lt[off_g + 1];
+                float p0 = 0.0f, p1 = 0.0f, p2 = 0.0f, p3 = 0.0f;
+#pragma unroll
+                for (int m = 0; m < R / 4; ++m) {
+                    if (EXACT || 4 * m < RL) {
+                        const float4 kk = k4[m], cq = q4[m];
+                        S[4 * m] = fmaf(kk.x, dtv, dec * S[4 * m]);
+                        S[4 * m + 1] = fmaf(kk.y, dtv, dec * S[4 * m + 1]);
+                        S[4 * m + 2] = fmaf(kk.z, dtv, dec * S[4 * m + 2]);
+                        S[4 * m + 3] = fmaf(kk.w, dtv, dec * S[4 * m + 3]);
+                        p0 = fmaf(S[4 * m], cq.x, p0);
+                        p1 = fmaf(S[4 * m + 1], cq.y, p1);
+                        p2 = fmaf(S[4 * m + 2], cq.z, p2);
+                        p3 = fmaf(S[4 * m + 3], cq.w, p3);
+                    }
+                }
+                o = fmaf(d_skip, vj, quad_sum((p0 + p1) + (p2 + p3)));
+            } else if (IS_DELTA) {
                 const float beta = lt[off_g], gdec = lt[off_g + 1];
                 float kn[R], qn[R];
                 float k2a = 0.0f, k2b = 0.0f, q2a = 0.0f, q2b = 0.0f;
@@ -249,8 +287,12 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
 #pragma unroll
                 for (int m = 0; m < R / 4; ++m) {
                     if (EXACT || 4 * m < RL) {
+                        if (KIND == SEQ_DELTA_CH) {  // one decay per key row
+                            const float4 ww = w4[m];
+                            S[4 * m] *= ww.x; S[4 * m + 1] *= ww.y; S[4 * m + 2] *= ww.z; S[4 * m + 3] *= ww.w;
+                        }
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) { kn[4 * m + e] *= kinv; S[4 * m + e] *= gdec; }
+                        for (int e = 0; e < 4; ++e) { kn[4 * m + e] *= kinv; if (KIND == SEQ_DELTA) S[4 * m + e] *= gdec; }
                         d0 = fmaf(S[4 * m], kn[4 * m], d0);
                         d1 = fmaf(S[4 * m + 1], kn[4 * m + 1], d1);
                         d2 = fmaf(S[4 * m + 2], kn[4 * m + 2], d2);
@@ -327,7 +369,7 @@ bool seq_recurrence_ok(int DK, int DV) { return DK >= 1 && DK <= SEQ_MAX_DK && D
 template <int KIND>
 static void seq_recurrence_launch(hipStream_t s, const seq_rec_args & a, int n_seqs) {
     const int RL = seq_rows_per_lane(a.DK);
-    const int per_tok = std::max(64, (KIND == SEQ_WKV6 ? 3 : 2) * SEQ_LPC * RL + SEQ_COLS + (KIND == SEQ_WKV6 ? 0 : 4));
+    const int per_tok = seq_per_tok(KIND, a.DK);
     int TB = std::max(1, std::min(SEQ_MAX_TB, SEQ_NV * 64 / per_tok));
     static const int tb_env = getenv("GGML_MI355X_SEQ_TB") ? atoi(getenv("GGML_MI355X_SEQ_TB")) : 0;  // (lab switch: fewer tokens per block)
     if (tb_env > 0) TB = std::min(TB, tb_env);
@@ -343,6 +385,8 @@ void launch_seq_recurrence(hipStream_t s, int kind, const seq_rec_args & a, int 
     if (n_seqs == 0 || a.H == 0) return;
     if (kind == SEQ_WKV6) seq_recurrence_launch<SEQ_WKV6>(s, a, n_seqs);
     else if (kind == SEQ_DELTA) seq_recurrence_launch<SEQ_DELTA>(s, a, n_seqs);
+    else if (kind == SEQ_DELTA_CH) seq_recurrence_launch<SEQ_DELTA_CH>(s, a, n_seqs);
+    else if (kind == SEQ_SSD) seq_recurrence_launch<SEQ_SSD>(s, a, n_seqs);
     else seq_recurrence_launch<SEQ_MLSTM>(s, a, n_seqs);
 }
 

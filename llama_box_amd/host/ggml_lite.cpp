@@ -612,6 +612,10 @@ struct ggml_tensor * ggml_seq_conv(struct ggml_context * ctx, struct ggml_tensor
     r->src[3] = taps > 1 ? hist : nullptr;
     return r;
 }
+void ggml_seq_conv_set_bias(struct ggml_tensor * conv, struct ggml_tensor * bias) {
+    LITE_ASSERT(conv->op == GGML_OP_SSM_CONV && conv->op_params[2] == 0 && bias->type == GGML_TYPE_F32 && ggml_nelements(bias) == conv->ne[0] * conv->ne[2]);
+    conv->src[4] = bias;
+}
 struct ggml_tensor * ggml_seq_conv_store(struct ggml_context * ctx, struct ggml_tensor * state, struct ggml_tensor * x, struct ggml_tensor * upd, struct ggml_tensor * info, int taps) {
     LITE_ASSERT(taps >= 2 && taps <= 16 && state->type == GGML_TYPE_F32 && state->ne[0] == x->ne[0] * (taps - 1) && upd->type == GGML_TYPE_I32 && info->type == GGML_TYPE_I32);
     LITE_ASSERT(upd->ne[0] >= taps - 1 && info->ne[0] == 4 && upd->ne[1] == info->ne[1]);
@@ -646,7 +650,10 @@ static ggml_tensor * seq_gla(ggml_context * ctx, int kind, ggml_tensor * q, ggml
                              ggml_tensor * info, int n_head, int n_head_k, float cap) {
     const int64_t DK = q->ne[0] / n_head_k, DV = v->ne[0] / n_head, T = q->ne[1];
     LITE_ASSERT(n_head % n_head_k == 0 && q->ne[0] == DK * n_head_k && k->ne[0] == q->ne[0] && v->ne[0] == DV * n_head && k->ne[1] == T && v->ne[1] == T);
-    LITE_ASSERT(gates->ne[0] == 2 * n_head && gates->ne[1] == T && ggml_nelements(params) == 2 * n_head && ggml_nelements(tok) == T && info->ne[0] == 4);
+    // raw gates per token and their parameters: two per head (delta rule, matrix memory), one per (head, key channel) with A_log per head in front of the offsets
+    // (channel decay), or one per head with (A_log, dt_bias, D) (state space)
+    const int64_t n_gates = kind == 3 ? DK * n_head : kind == 4 ? n_head : 2 * n_head, n_par = kind == 3 ? n_head + DK * n_head : kind == 4 ? 3 * n_head : 2 * n_head;
+    LITE_ASSERT(gates->ne[0] == n_gates && gates->ne[1] == T && ggml_nelements(params) == n_par && ggml_nelements(tok) == T && info->ne[0] == 4);
     LITE_ASSERT(state->ne[0] == ggml_seq_state_size(kind, n_head, (int) DK, (int) DV));
     ggml_tensor * o = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, DV, n_head, T);
     o->op = GGML_OP_GATED_LINEAR_ATTN;
@@ -663,6 +670,17 @@ static ggml_tensor * seq_gla(ggml_context * ctx, int kind, ggml_tensor * q, ggml
 struct ggml_tensor * ggml_seq_gated_delta(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * ba, struct ggml_tensor * adt,
                                           struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, int n_head_k) {
     return seq_gla(ctx, 1, q, k, v, ba, adt, state, tok, info, n_head, n_head_k, 0.0f);
+}
+struct ggml_tensor * ggml_seq_delta_channel(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * b_pre, struct ggml_tensor * a_pre,
+                                            struct ggml_tensor * a_dt, struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, int n_head_k) {
+    LITE_ASSERT(b_pre->type == GGML_TYPE_F32 && b_pre->ne[0] == n_head && b_pre->ne[1] == q->ne[1]);
+    ggml_tensor * o = seq_gla(ctx, 3, q, k, v, a_pre, a_dt, state, tok, info, n_head, n_head_k, 0.0f);
+    o->src[8] = b_pre;
+    return o;
+}
+struct ggml_tensor * ggml_seq_ssd(struct ggml_context * ctx, struct ggml_tensor * c, struct ggml_tensor * b, struct ggml_tensor * x, struct ggml_tensor * dt_pre, struct ggml_tensor * a_dt_d,
+                                  struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, int n_group) {
+    return seq_gla(ctx, 4, c, b, x, dt_pre, a_dt_d, state, tok, info, n_head, n_group, 0.0f);
 }
 struct ggml_tensor * ggml_seq_mlstm(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * if_pre, struct ggml_tensor * if_bias,
                                     struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, float cap) {

@@ -126,6 +126,8 @@ struct ggml_tensor * ggml_argmax(struct ggml_context * ctx, struct ggml_tensor *
    one column per slot, and are updated IN PLACE by the ops. */
 /* y[c, t, m] = act(sum_j w[j, c, m] x_(t - (taps - 1 - j))[c]): x [C, T], w [taps, C, M], state [C (taps - 1), slots] (NULL when taps == 1); act 0 none, 1 SiLU */
 struct ggml_tensor * ggml_seq_conv(struct ggml_context * ctx, struct ggml_tensor * x, struct ggml_tensor * w, struct ggml_tensor * state, struct ggml_tensor * hist, int act);
+/* a bias [C, M] added to the convolution's sum before the activation */
+void ggml_seq_conv_set_bias(struct ggml_tensor * conv, struct ggml_tensor * bias);
 /* the last taps - 1 inputs of every sequence of the batch become its state; returns (a view of) the state */
 struct ggml_tensor * ggml_seq_conv_store(struct ggml_context * ctx, struct ggml_tensor * state, struct ggml_tensor * x, struct ggml_tensor * upd, struct ggml_tensor * info, int taps);
 /* per head o_t = (S + diag(u) k v^T)^T r, then S <- diag(w) S + k v^T with w = exp(-exp(w_pre + w0)): r, k, v, w_pre [D H, T]; w0, u [D H] -> [D, H, T] */
@@ -135,12 +137,20 @@ struct ggml_tensor * ggml_seq_wkv6(struct ggml_context * ctx, struct ggml_tensor
    g = exp(-exp(A_log) softplus(a_pre + dt_bias)): q, k [DK G, T]; v [DV H, T]; ba [2 H, T] (b_pre, a_pre); adt [2 H] (A_log, dt_bias) -> [DV, H, T] */
 struct ggml_tensor * ggml_seq_gated_delta(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * ba, struct ggml_tensor * adt,
                                           struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, int n_head_k);
+/* the gated delta rule with one decay per (head, key channel): S <- diag(g) S with g = exp(-exp(A_log_h) softplus(a_pre + dt_bias)), the rest as ggml_seq_gated_delta:
+   q, k [DK G, T]; v [DV H, T]; b_pre [H, T]; a_pre [DK H, T]; a_dt [H + DK H] (A_log of every head, then dt_bias of every (head, channel)) -> [DV, H, T] */
+struct ggml_tensor * ggml_seq_delta_channel(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * b_pre, struct ggml_tensor * a_pre,
+                                            struct ggml_tensor * a_dt, struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, int n_head_k);
+/* state-space duality (Mamba-2) per head: dt = softplus(dt_pre + dt_bias); S <- exp(-exp(A_log) dt) S + dt b x^T (S is N x DV); y = S^T c + D x; head h reads group
+   h / (H / G) of b and c: c, b [N G, T]; x [DV H, T]; dt_pre [H, T]; a_dt_d [3 H] (A_log, dt_bias, D) -> [DV, H, T] */
+struct ggml_tensor * ggml_seq_ssd(struct ggml_context * ctx, struct ggml_tensor * c, struct ggml_tensor * b, struct ggml_tensor * x, struct ggml_tensor * dt_pre, struct ggml_tensor * a_dt_d,
+                                  struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, int n_group);
 /* matrix memory with exponential gates under a running maximum: i = cap tanh((i_pre + b_i) / cap), f = log sigmoid(cap tanh((f_pre + b_f) / cap)); m' = max(f + m, i);
    S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k alone; o = S^T q / (max(|n . q|, e^(-m')) + 1e-6), q times dk^-1/2: q, k [DK H, T]; v [DV H, T];
    if_pre [2 H, T]; if_bias [2 H] -> [DV, H, T] */
 struct ggml_tensor * ggml_seq_mlstm(struct ggml_context * ctx, struct ggml_tensor * q, struct ggml_tensor * k, struct ggml_tensor * v, struct ggml_tensor * if_pre, struct ggml_tensor * if_bias,
                                     struct ggml_tensor * state, struct ggml_tensor * tok, struct ggml_tensor * info, int n_head, float cap);
-/* f32 values of state one slot of a recurrence holds (kind: 0 wkv6, 1 gated delta, 2 mlstm) */
+/* f32 values of state one slot of a recurrence holds (kind: 0 wkv6, 1 gated delta, 2 mlstm, 3 delta with channel decay, 4 state space) */
 int64_t ggml_seq_state_size(int kind, int n_head, int dk, int dv);
 
 /* graphs */

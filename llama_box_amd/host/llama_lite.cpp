@@ -343,12 +343,21 @@ struct llm_layer {
     ggml_tensor *wqkv = nullptr, *bqkv = nullptr, *conv = nullptr, *wgates = nullptr, *gate_par = nullptr, *sub_norm = nullptr, *bo = nullptr, *attn_fb = nullptr;
     ggml_tensor *tm_taps = nullptr, *tm_rkvg = nullptr, *tm_w1 = nullptr, *tm_w2 = nullptr, *tm_w0 = nullptr, *tm_u = nullptr, *tm_norm = nullptr, *tm_out = nullptr;
     ggml_tensor *ffn_gate_up_exps = nullptr;
+    // ... a query latent in front of the query heads (down projection, its norm); the weights of a per-head norm on queries and keys (one row shared by the heads)
+    ggml_tensor *wdq = nullptr, *dq_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
+    // ... a delta rule with one decay per key channel beside an attention (its own q, k, v as one projection in wqkv / conv; beta; the decay and the output gate through
+    // two small matrices each; its output projection) and the norm weights of the two branches' outputs
+    ggml_tensor *wbeta = nullptr, *wa1 = nullptr, *wa2 = nullptr, *wg1 = nullptr, *wg2 = nullptr, *wo_r = nullptr, *left_norm = nullptr, *right_norm = nullptr;
+    // ... a state-space mixer: the input projection in three parts (gate z, convolved (x, B, C), step sizes), the convolution's bias
+    ggml_tensor *ssm_in_z = nullptr, *ssm_in_xbc = nullptr, *ssm_in_dt = nullptr, *conv_b = nullptr;
+    // ... a per-layer token input: the layer's part of a second embedding table, a gate on the stream, the projection back and the norm weight
+    ggml_tensor *side_embd = nullptr, *side_gate = nullptr, *side_proj = nullptr, *side_norm = nullptr;
 };
 
 // one layer of a model whose config lists its layers one by one (sizes and constants may differ from layer to layer)
 enum llm_mlp_kind { LLM_MLP_NONE = 0, LLM_MLP_DENSE = 1, LLM_MLP_MOE = 2 };
 // (from LLM_MIX_MLSTM on: mixers that keep state per sequence and bring their own output projection)
-enum llm_mixer_kind { LLM_MIX_ATTN = 0, LLM_MIX_LATENT = 1, LLM_MIX_MLSTM = 2, LLM_MIX_DELTA = 3, LLM_MIX_SIGMOID_WKV = 4 };
+enum llm_mixer_kind { LLM_MIX_ATTN = 0, LLM_MIX_LATENT = 1, LLM_MIX_MLSTM = 2, LLM_MIX_DELTA = 3, LLM_MIX_SIGMOID_WKV = 4, LLM_MIX_SSD = 5, LLM_MIX_ATTN_DELTA = 6 };
 struct llm_layer_cfg {
     int n_head = 0, n_head_kv = 0, dk = 0, dv = 0;  // query heads, key/value heads, per-head query/key size, per-head value size
     int rot_dims = 0;                               // leading dims of every head that are rotated, as neighbouring pairs
@@ -387,6 +396,14 @@ struct llm_layer_cfg {
     bool moe_scores_all = false;
     int moe_groups = 1, moe_keep = 1;
     float moe_scale = 1.0f;
+    bool two_norms = false;                         // with `parallel`: x += mixer(norm1(x)) + ff(norm2(x)), two norms of the same x
+    bool ffn_relu_sq = false;                       // dense feed-forward W_down relu(W_up h)^2
+    bool qk_norm = false;                           // queries and keys are RMS-normed per head with a weight row shared by the heads
+    int q_rank = 0;                                 // > 0: queries come through a normed latent of this size
+    int kv_from = -1;                               // >= 0: a latent-attention layer without a down projection of its own, reading that layer's cache rows
+    int ssm_state = 0, ssm_groups = 1, ssm_norm_groups = 1;  // state-space mixer (LLM_MIX_SSD): state size per head, groups of (B, C), parts of the gated norm; n_head x dv = inner
+    int r_head = 0, r_head_kv = 0, r_dk = 0, r_dv = 0, r_rank = 0;  // the delta rule beside an attention (LLM_MIX_ATTN_DELTA): heads, key heads, sizes, inner size of decay / gate
+    int side_dim = 0;                               // > 0: the per-layer token input of this many entries
 };
 // what a layer's positions may see: one attention mask per distinct rule of a model
 struct llm_mask_rule {
@@ -815,6 +832,9 @@ struct dir_tensor {               // one framework tensor and where its values c
     float synth_lo = 0.0f, synth_hi = 0.0f;  // random weights: uniform in [lo, hi) when hi > lo (shift factors, penalties)
     bool broadcast = false;       // the checkpoint holds ONE number: every entry of the tensor gets it (a norm with a scalar weight)
     bool mix_taps = false;        // src are token-shift factors mu [ne1] each: kept as 2-tap convolution weights (mu for the previous token, 1 - mu for the token's own), [2, ne1, n_src]
+    bool one_plus = false;        // a norm weight stored around zero: 1 is added to every entry (f32 tensors)
+    int64_t row0 = -1;            // >= 0: the ONE source is [rows, ne0] and rows row0 .. row0 + ne1 - 1 of it are taken (a projection stored as one matrix, kept in parts)
+    int64_t col0 = -1;            // >= 0: the ONE source is [ne1, columns] and columns col0 .. col0 + ne0 - 1 of every row are taken (a layer's part of a shared table)
 };
 
 // the visibility rule of a layer gets a mask of its own unless another layer has the same
@@ -1305,6 +1325,210 @@ static std::vector<dir_tensor> nigozen_plan(const llm_model * m) {
     return plan;
 }
 
+// Nogavik: every layer is x += mixer(norm1(x)) + ff(norm2(x)) — two RMS norms of the same x whose weights are stored around zero (the loader adds 1) — followed by a
+// per-layer token input: the layer's part e of a second embedding table, y = W_proj (gelu_tanh(W_gate x) * e), x += rms_norm(y) * w.  Mixers: latent attention whose
+// queries come through a normed latent as well, neighbouring rotation pairs, a sigmoid output gate per value entry, and optionally the cache rows of an earlier layer
+// instead of a down projection of its own (kv_from); a state-space mixer (Mamba-2); grouped-query attention with biases and per-head normed queries and keys (no
+// rotation) beside a gated delta rule with one decay per key channel, the two outputs RMS-normed over the width and averaged.  Dense feed-forward with squared ReLU.
+// The output matrix is the embedding table.
+static bool parse_nogavik_config(const json_value & cfg, const st_file * file, llm_model * m, std::string & err) {
+    llm_hparams & hp = m->hp;
+    snprintf(hp.arch, sizeof(hp.arch), "nogavik");
+    const json_value * layers = cfg.get("layers");
+    if (!layers || layers->kind != json_value::ARR || layers->arr.empty()) { err = "config: no layers"; return false; }
+    const json_value * v;
+    hp.n_embd = (v = cfg.get("width")) ? (int) v->number(0) : 0;
+    hp.n_vocab = (v = cfg.get("vocab")) ? (int) v->number(0) : 0;
+    hp.rms_eps = (v = cfg.path("norm", "eps")) ? (float) v->number(1e-5) : 1e-5f;
+    hp.n_layer = (int) layers->arr.size();
+    hp.n_ctx_train = 1 << 20;
+    if (hp.n_embd <= 0 || hp.n_vocab <= 0) { err = "config: width / vocab missing"; return false; }
+    auto num = [&](const json_value * o, const char * k0, const char * k1, double d) { const json_value * x = o->path(k0, k1); return x ? x->number(d) : d; };
+    const int side_dim = (v = cfg.path("token_side", "dim")) ? (int) v->number(0) : 0;
+    if (side_dim < 0) { err = "config: inconsistent token_side"; return false; }
+    m->lcfg.resize((size_t) hp.n_layer);
+    m->has_attn = false;
+    m->has_seq_state = false;
+    m->hist_rows = 0;
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const json_value & L = layers->arr[(size_t) il];
+        llm_layer_cfg & c = m->lcfg[(size_t) il];
+        const std::string lname = "config: layer " + std::to_string(il);
+        const json_value * type = L.get("type");
+        const json_value * mx = L.get("mixer");
+        if (!type || type->kind != json_value::STR || !mx || mx->kind != json_value::OBJ) { err = lname + ": no mixer"; return false; }
+        c.rms = c.parallel = c.two_norms = true;
+        c.side_dim = side_dim;
+        c.rot_dims = 0;
+        if (type->str == "latent_attention") {
+            c.mixer = LLM_MIX_LATENT;
+            c.n_head = (int) num(mx, "heads", nullptr, 0);
+            c.n_head_kv = 1;
+            c.dk = (int) num(mx, "dim", nullptr, 0);
+            c.dv = (int) num(mx, "vdim", nullptr, c.dk);
+            c.kv_rank = (int) num(mx, "kv_rank", nullptr, 0);
+            c.q_rank = (int) num(mx, "q_rank", nullptr, 0);
+            c.rot_dim = (int) num(mx, "rot_dim", nullptr, 0);
+            c.rot_dims = c.rot_dim;  // the rotated vector is the rot_dim part of a head, all of it
+            c.rot_half = false;      // pairs are neighbours (2i, 2i + 1)
+            c.rot_base = (float) num(mx, "rot", "base", 10000.0);
+            c.scale = (float) num(mx, "scale", nullptr, c.dk + c.rot_dim > 0 ? 1.0 / sqrt((double) (c.dk + c.rot_dim)) : 1.0);
+            c.out_gate = true;
+            if (const json_value * kf = mx->path("kv_from")) c.kv_from = (int) kf->number(-1);
+            if (c.n_head <= 0 || c.dk <= 0 || c.dv <= 0 || c.kv_rank <= 0 || c.q_rank <= 0 || c.rot_dim < 0 || (c.rot_dim & 1)) { err = lname + ": inconsistent latent attention sizes"; return false; }
+            if (num(mx, "rot", "dims", c.rot_dim) != c.rot_dim) { err = lname + ": rot.dims differs from rot_dim"; return false; }
+            if (mx->get("kv_from") && mx->get("kv_from")->kind != json_value::NUL) {
+                const llm_layer_cfg * o = c.kv_from >= 0 && c.kv_from < il ? &m->lcfg[(size_t) c.kv_from] : nullptr;
+                if (!o || o->mixer != LLM_MIX_LATENT || o->kv_from >= 0 || o->kv_rank != c.kv_rank || o->rot_dim != c.rot_dim || o->rot_base != c.rot_base) {
+                    err = lname + ": kv_from names no earlier latent-attention layer with a down projection of its own and the same latent, rotated part and rotation";
+                    return false;
+                }
+            }
+            m->has_attn = true;
+            m->max_embd_k = std::max(m->max_embd_k, c.kv_rank + c.rot_dim);
+        } else if (type->str == "mamba2") {
+            c.mixer = LLM_MIX_SSD;
+            c.n_head = (int) num(mx, "heads", nullptr, 0);
+            c.dv = (int) num(mx, "vdim", nullptr, 0);
+            c.ssm_state = c.dk = (int) num(mx, "state", nullptr, 0);
+            c.ssm_groups = c.n_head_kv = (int) num(mx, "groups", nullptr, 1);
+            c.ssm_norm_groups = (int) num(mx, "norm_groups", nullptr, 1);
+            c.conv_taps = (int) num(mx, "conv", nullptr, 1);
+            if (c.n_head <= 0 || c.dv <= 0 || c.ssm_state <= 0 || c.ssm_state > 256 || c.ssm_groups <= 0 || c.n_head % c.ssm_groups || c.ssm_norm_groups <= 0 ||
+                (c.n_head * c.dv) % c.ssm_norm_groups || c.conv_taps < 1 || c.conv_taps > 16) { err = lname + ": inconsistent state-space sizes"; return false; }
+            m->has_seq_state = true;
+        } else if (type->str == "parallel") {
+            c.mixer = LLM_MIX_ATTN_DELTA;
+            const json_value * lf = mx->get("left"), * rt = mx->get("right");
+            if (!lf || lf->kind != json_value::OBJ || !rt || rt->kind != json_value::OBJ) { err = lname + ": a parallel mixer needs left and right"; return false; }
+            c.n_head = (int) num(lf, "heads", nullptr, 0);
+            c.n_head_kv = (int) num(lf, "kv_heads", nullptr, c.n_head);
+            c.dk = (int) num(lf, "dim", nullptr, 0);
+            c.dv = (int) num(lf, "vdim", nullptr, c.dk);
+            c.scale = (float) num(lf, "scale", nullptr, c.dk > 0 ? 1.0 / sqrt((double) c.dk) : 1.0);
+            c.qkv_bias = c.qk_norm = true;
+            c.left_scale = c.right_scale = 0.5f;
+            c.r_head = (int) num(rt, "heads", nullptr, 0);
+            c.r_head_kv = (int) num(rt, "kv_heads", nullptr, c.r_head);
+            c.r_dk = (int) num(rt, "dim", nullptr, 0);
+            c.r_dv = (int) num(rt, "vdim", nullptr, c.r_dk);
+            c.conv_taps = (int) num(rt, "conv", nullptr, 1);
+            c.r_rank = (int) num(rt, "rank", nullptr, 16);  // (a checkpoint's a1 gives it)
+            if (file) {
+                const st_tensor * a1 = file->find("l" + std::to_string(il) + ".mix.right.a1");
+                if (!a1 || a1->shape.size() != 2) { err = lname + ": no right.a1 in the checkpoint"; return false; }
+                c.r_rank = (int) a1->shape[0];
+            }
+            if (c.n_head <= 0 || c.n_head_kv <= 0 || c.n_head % c.n_head_kv || c.dk <= 0 || c.dv <= 0 || c.r_head <= 0 || c.r_head_kv <= 0 || c.r_head % c.r_head_kv || c.r_dk <= 0 ||
+                c.r_dk > 256 || c.r_dv <= 0 || c.r_rank <= 0 || c.conv_taps < 1 || c.conv_taps > 16) { err = lname + ": inconsistent parallel-mixer sizes"; return false; }
+            m->has_attn = true;
+            m->has_seq_state = true;
+            m->max_embd_k = std::max(m->max_embd_k, c.n_head_kv * c.dk);
+            m->max_embd_v = std::max(m->max_embd_v, c.n_head_kv * c.dv);
+        } else { err = lname + ": unknown mixer type"; return false; }
+        m->hist_rows = std::max(m->hist_rows, c.conv_taps - 1);
+        c.mask_id = mask_rule_id(m, llm_mask_rule());  // every attention of the design is plainly causal
+        const json_value * ml = L.path("mlp");
+        if (ml && ml->kind == json_value::OBJ) {
+            const json_value * kind = ml->get("kind");
+            if (!kind || kind->kind != json_value::STR || kind->str != "dense") { err = lname + ": unknown mlp kind"; return false; }
+            c.mlp = LLM_MLP_DENSE;
+            c.ffn_relu_sq = true;
+            c.n_ff = (int) num(ml, "ff", nullptr, 0);
+            if (c.n_ff <= 0) { err = lname + ": ff missing"; return false; }
+        }
+    }
+    hp.n_head = m->lcfg[0].n_head; hp.n_head_kv = m->lcfg[0].n_head_kv; hp.n_embd_head = m->lcfg[0].dk; hp.n_ff = m->lcfg[0].n_ff;
+    hp.rope_freq_base = m->lcfg[0].rot_base;
+    for (int il = 0; il < hp.n_layer; ++il) m->runs.push_back({il, -1, false});
+    return true;
+}
+
+static std::vector<dir_tensor> nogavik_plan(const llm_model * m) {
+    const llm_hparams & hp = m->hp;
+    const ggml_type wt = m->wtype;
+    const int64_t E = hp.n_embd;
+    std::vector<dir_tensor> plan;
+    auto add = [&](const std::string & name, ggml_type t, int64_t n0, int64_t n1, int64_t n2, std::vector<std::string> src, float gain) -> dir_tensor & {
+        dir_tensor d;
+        d.name = name; d.type = t; d.ne[0] = n0; d.ne[1] = n1; d.ne[2] = n2; d.src = std::move(src); d.synth_gain = gain;
+        plan.push_back(std::move(d));
+        return plan.back();
+    };
+    auto uniform = [&](dir_tensor & t, float lo, float hi) -> dir_tensor & { t.synth_lo = lo; t.synth_hi = hi; return t; };
+    auto norm1p = [&](const std::string & name, const std::string & src) { uniform(add(name, GGML_TYPE_F32, E, 1, 1, {src}, 0.0f), -0.2f, 0.3f).one_plus = true; };  // 1 + w
+    auto normw = [&](const std::string & name, int64_t n, const std::string & src) { uniform(add(name, GGML_TYPE_F32, n, 1, 1, {src}, 0.0f), 0.7f, 1.4f); };           // plain weight
+    add("token_embd.weight", wt, E, hp.n_vocab, 1, {"embed"}, sqrtf((float) E));
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const llm_layer_cfg & c = m->lcfg[(size_t) il];
+        const std::string p = "blk." + std::to_string(il) + ".", q = "l" + std::to_string(il) + ".", x = q + "mix.";
+        const int64_t H = c.n_head, G = c.n_head_kv;
+        norm1p(p + "attn_norm.weight", q + "norm1");
+        if (c.mixer == LLM_MIX_LATENT) {
+            add(p + "attn_q_a.weight", wt, E, c.q_rank, 1, {x + "dq"}, 1.0f);
+            normw(p + "attn_q_a_norm.weight", c.q_rank, x + "dq.norm");
+            add(p + "attn_q.weight", wt, c.q_rank, H * (c.dk + c.rot_dim), 1, {x + "uq"}, 2.0f);
+            if (c.kv_from < 0) {
+                add(p + "attn_kv_a.weight", wt, E, c.kv_rank + c.rot_dim, 1, {x + "dkv"}, 1.0f);
+                normw(p + "attn_kv_a_norm.weight", c.kv_rank, x + "dkv.norm");
+            }
+            add(p + "attn_k_b_t.weight", wt, c.dk, c.kv_rank, H, {x + "uk"}, 1.0f).head_transpose = true;
+            add(p + "attn_v_b.weight", wt, c.kv_rank, c.dv, H, {x + "uv"}, 1.0f);
+            if (c.rot_dim > 0) add(p + "rope_freq.weight", GGML_TYPE_F32, c.rot_dim / 2, 1, 1, {}, 0.0f).values = rope_frequencies(c);
+            add(p + "attn_gate.weight", wt, E, H * c.dv, 1, {x + "g"}, 1.0f);
+            add(p + "attn_output.weight", wt, H * c.dv, E, 1, {x + "o"}, 1.0f);
+        } else if (c.mixer == LLM_MIX_SSD) {
+            const int64_t inner = H * c.dv, GN = (int64_t) c.ssm_groups * c.ssm_state, ch = inner + 2 * GN;
+            // the input projection [z | x, B, C | dt] is kept in its three parts: each is read whole by what follows it
+            add(p + "ssm_in_z.weight", wt, E, inner, 1, {x + "in"}, 1.0f).row0 = 0;
+            add(p + "ssm_in_xbc.weight", wt, E, ch, 1, {x + "in"}, 2.0f).row0 = inner;
+            add(p + "ssm_in_dt.weight", wt, E, H, 1, {x + "in"}, 2.0f).row0 = inner + ch;
+            add(p + "ssm_conv1d.weight", GGML_TYPE_F32, c.conv_taps, ch, 1, {x + "conv"}, 1.0f);
+            add(p + "ssm_conv1d.bias", GGML_TYPE_F32, ch, 1, 1, {x + "conv.b"}, 0.3f * sqrtf((float) ch));
+            uniform(add(p + "ssm_params.weight", GGML_TYPE_F32, 3 * H, 1, 1, {x + "A_log", x + "dt_bias", x + "D"}, 0.0f), -1.5f, 0.5f);
+            normw(p + "attn_sub_norm.weight", inner, x + "norm");
+            add(p + "attn_output.weight", wt, inner, E, 1, {x + "o"}, 1.0f);
+        } else {
+            const std::string l = x + "left.", r = x + "right.";
+            add(p + "attn_q.weight", wt, E, H * c.dk, 1, {l + "q"}, 2.0f);
+            add(p + "attn_k.weight", wt, E, G * c.dk, 1, {l + "k"}, 2.0f);
+            add(p + "attn_v.weight", wt, E, G * c.dv, 1, {l + "v"}, 1.0f);
+            add(p + "attn_q.bias", GGML_TYPE_F32, H * c.dk, 1, 1, {l + "q.b"}, 0.3f * sqrtf((float) (H * c.dk)));
+            add(p + "attn_k.bias", GGML_TYPE_F32, G * c.dk, 1, 1, {l + "k.b"}, 0.3f * sqrtf((float) (G * c.dk)));
+            add(p + "attn_v.bias", GGML_TYPE_F32, G * c.dv, 1, 1, {l + "v.b"}, 0.3f * sqrtf((float) (G * c.dv)));
+            normw(p + "attn_q_norm.weight", c.dk, l + "q.norm");
+            normw(p + "attn_k_norm.weight", c.dk, l + "k.norm");
+            add(p + "attn_output.weight", wt, H * c.dv, E, 1, {l + "o"}, 1.0f);
+            normw(p + "mix_left_norm.weight", E, l + "out");
+            const int64_t RH = c.r_head, RG = c.r_head_kv, C = 2 * RG * c.r_dk + RH * c.r_dv;
+            add(p + "attn_qkv.weight", wt, E, C, 1, {r + "q", r + "k", r + "v"}, 2.0f);
+            add(p + "ssm_conv1d.weight", GGML_TYPE_F32, c.conv_taps, C, 1, {r + "q.conv", r + "k.conv", r + "v.conv"}, 1.0f);
+            add(p + "delta_beta.weight", wt, E, RH, 1, {r + "b"}, 2.0f);
+            add(p + "delta_a1.weight", wt, E, c.r_rank, 1, {r + "a1"}, 1.0f);
+            add(p + "delta_a2.weight", wt, c.r_rank, RH * c.r_dk, 1, {r + "a2"}, 2.0f);
+            uniform(add(p + "attn_gates.param", GGML_TYPE_F32, RH + RH * c.r_dk, 1, 1, {r + "A_log", r + "dt_bias"}, 0.0f), -1.5f, 0.5f);
+            add(p + "delta_g1.weight", wt, E, c.r_rank, 1, {r + "g1"}, 1.0f);
+            add(p + "delta_g2.weight", wt, c.r_rank, RH * c.r_dv, 1, {r + "g2"}, 2.0f);
+            normw(p + "attn_sub_norm.weight", c.r_dv, r + "norm");
+            add(p + "delta_output.weight", wt, RH * c.r_dv, E, 1, {r + "o"}, 1.0f);
+            normw(p + "mix_right_norm.weight", E, r + "out");
+        }
+        if (c.mlp == LLM_MLP_DENSE) {
+            norm1p(p + "ffn_norm.weight", q + "norm2");
+            add(p + "ffn_up.weight", wt, E, c.n_ff, 1, {q + "mlp.up"}, 1.4f);
+            add(p + "ffn_down.weight", wt, c.n_ff, E, 1, {q + "mlp.down"}, 1.0f);
+        }
+        if (c.side_dim > 0) {
+            add(p + "side_embd.weight", wt, c.side_dim, hp.n_vocab, 1, {"side.embed"}, sqrtf((float) c.side_dim)).col0 = (int64_t) il * c.side_dim;
+            add(p + "side_gate.weight", wt, E, c.side_dim, 1, {q + "side.gate"}, 1.0f);
+            add(p + "side_proj.weight", wt, c.side_dim, E, 1, {q + "side.proj"}, 1.0f);
+            normw(p + "side_norm.weight", E, q + "side.norm");
+        }
+    }
+    norm1p("output_norm.weight", "final.norm");
+    return plan;
+}
+
 // values of one checkpoint tensor (bf16 / f32 / f16 in the file) as `type` (bf16 or f32) into dst
 static bool convert_values(const st_tensor & t, ggml_type type, uint8_t * dst) {
     const int64_t n = t.numel();
@@ -1343,6 +1567,9 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
     } else if (arch->str == "Rarelorn") {
         if (!parse_rarelorn_config(cfg, file, m, err)) { fprintf(stderr, "llm_model_load_dir: %s\n", err.c_str()); delete m; return nullptr; }
         plan = rarelorn_plan(m);
+    } else if (arch->str == "Nogavik") {
+        if (!parse_nogavik_config(cfg, file, m, err)) { fprintf(stderr, "llm_model_load_dir: %s\n", err.c_str()); delete m; return nullptr; }
+        plan = nogavik_plan(m);
     } else {
         fprintf(stderr, "llm_model_load_dir: unknown architecture \"%s\"\n", arch->str.c_str());
         delete m;
@@ -1351,7 +1578,17 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
     m->ctx = ggml_init({0, nullptr, true});
     for (auto & t : plan) {
         // shapes are checked against the file before anything is allocated
-        if (file && (t.broadcast || t.mix_taps || (t.src.size() > 1 && t.ne[2] == 1))) {
+        if (file && (t.row0 >= 0 || t.col0 >= 0)) {
+            // a part of ONE stored matrix: some of its rows, or some columns of every row
+            const st_tensor * st = t.src.size() == 1 ? file->find(t.src[0]) : nullptr;
+            const bool ok = st && st->shape.size() == 2 && t.ne[2] == 1 &&
+                            (t.row0 >= 0 ? st->shape[1] == t.ne[0] && t.row0 + t.ne[1] <= st->shape[0] : st->shape[0] == t.ne[1] && t.col0 + t.ne[0] <= st->shape[1]);
+            if (!ok) {
+                fprintf(stderr, "llm_model_load_dir: tensor %s (a part of %s) is missing or has another shape than the config implies\n", t.name.c_str(), t.src.empty() ? "?" : t.src[0].c_str());
+                llm_model_free(m);
+                return nullptr;
+            }
+        } else if (file && (t.broadcast || t.mix_taps || (t.src.size() > 1 && t.ne[2] == 1))) {
             // one number for a whole row; shift factors of ne1 entries each; or matrices / vectors of UNEQUAL heights stacked along dim 1 (q, k, v as one projection)
             int64_t total = 0;
             bool ok = true;
@@ -1399,6 +1636,12 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
             memcpy(stage.data(), t.values.data(), total);
         } else if (t.src.empty()) {
             // zeros (the sinks)
+        } else if (file && (t.row0 >= 0 || t.col0 >= 0)) {
+            const st_tensor * st = file->find(t.src[0]);
+            std::vector<uint8_t> whole((size_t) st->numel() * esz);
+            if (!convert_values(*st, t.type, whole.data())) { fprintf(stderr, "llm_model_load_dir: tensor %s has an unsupported dtype\n", t.src[0].c_str()); llm_model_free(m); return nullptr; }
+            if (t.row0 >= 0) memcpy(stage.data(), whole.data() + (size_t) (t.row0 * t.ne[0]) * esz, total);
+            else for (int64_t r = 0; r < t.ne[1]; ++r) memcpy(stage.data() + (size_t) (r * t.ne[0]) * esz, whole.data() + (size_t) (r * st->shape[1] + t.col0) * esz, (size_t) t.ne[0] * esz);
         } else if (file && (t.broadcast || t.mix_taps)) {
             LLM_ASSERT(t.type == GGML_TYPE_F32);
             float * out = (float *) stage.data();
@@ -1460,6 +1703,11 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
                 else { const uint16_t h = f32_to_bf16(f); memcpy(stage.data() + i * 2, &h, 2); }
             }
         }
+        if (t.one_plus) {  // (the sum is rounded to f32 once, here)
+            LLM_ASSERT(t.type == GGML_TYPE_F32);
+            float * out = (float *) stage.data();
+            for (int64_t i = 0; i < t.ne[0] * t.ne[1] * t.ne[2]; ++i) out[i] += 1.0f;
+        }
         ggml_backend_tensor_set(x, stage.data(), 0, stage.size());
         m->total_bytes += stage.size();
     }
@@ -1493,11 +1741,21 @@ static llm_model * model_from_config(const json_value & cfg, const st_file * fil
         L.gate_par = g("attn_gates.bias") ? g("attn_gates.bias") : g("attn_gates.param"); L.sub_norm = g("attn_sub_norm.weight"); L.bo = g("attn_output.bias"); L.attn_fb = g("attn_fb.weight");
         L.tm_taps = g("time_mix_taps.weight"); L.tm_rkvg = g("time_mix_rkvg.weight"); L.tm_w1 = g("time_mix_w1.weight"); L.tm_w2 = g("time_mix_w2.weight"); L.tm_w0 = g("time_mix_w0.weight");
         L.tm_u = g("time_mix_first.weight"); L.tm_norm = g("time_mix_ln.weight"); L.tm_out = g("time_mix_output.weight"); L.ffn_gate_up_exps = g("ffn_gate_up_exps.weight");
+        L.bq = g("attn_q.bias"); L.bk = g("attn_k.bias"); L.bv = g("attn_v.bias"); L.q_norm = g("attn_q_norm.weight"); L.k_norm = g("attn_k_norm.weight");
+        L.wdq = g("attn_q_a.weight"); L.dq_norm = g("attn_q_a_norm.weight");
+        L.wbeta = g("delta_beta.weight"); L.wa1 = g("delta_a1.weight"); L.wa2 = g("delta_a2.weight"); L.wg1 = g("delta_g1.weight"); L.wg2 = g("delta_g2.weight");
+        L.wo_r = g("delta_output.weight"); L.left_norm = g("mix_left_norm.weight"); L.right_norm = g("mix_right_norm.weight");
+        L.ssm_in_z = g("ssm_in_z.weight"); L.ssm_in_xbc = g("ssm_in_xbc.weight"); L.ssm_in_dt = g("ssm_in_dt.weight"); L.conv_b = g("ssm_conv1d.bias");
+        if (!L.gate_par) L.gate_par = g("ssm_params.weight");
+        L.side_embd = g("side_embd.weight"); L.side_gate = g("side_gate.weight"); L.side_proj = g("side_proj.weight"); L.side_norm = g("side_norm.weight");
         L.wdkv = g("attn_kv_a.weight"); L.dkv_norm = g("attn_kv_a_norm.weight"); L.wuk_t = g("attn_k_b_t.weight"); L.wuv = g("attn_v_b.weight"); L.rope_freq = g("rope_freq.weight");
         for (ggml_tensor * t : {L.attn_norm, L.attn_post_norm, L.wq, L.wk, L.wv, L.attn_gate, L.wo, L.ffn_norm, L.ffn_post_norm, L.ffn_up, L.ffn_down, L.ffn_gate_inp,
                                 L.attn_sink, L.attn_r12, L.shift, L.ffn_gate, L.ffn_gate_b, L.ffn_up_b, L.ffn_down_b, L.wdkv, L.dkv_norm, L.wuk_t, L.wuv, L.rope_freq,
-                                L.wqkv, L.bqkv, L.conv, L.wgates, L.gate_par, L.sub_norm, L.bo, L.attn_fb, L.tm_taps, L.tm_rkvg, L.tm_w1, L.tm_w2, L.tm_w0, L.tm_u, L.tm_norm, L.tm_out})
+                                L.wqkv, L.bqkv, L.conv, L.wgates, L.gate_par, L.sub_norm, L.bo, L.attn_fb, L.tm_taps, L.tm_rkvg, L.tm_w1, L.tm_w2, L.tm_w0, L.tm_u, L.tm_norm, L.tm_out,
+                                L.bq, L.bk, L.bv, L.q_norm, L.k_norm, L.wdq, L.dq_norm, L.wbeta, L.wa1, L.wa2, L.wg1, L.wg2, L.wo_r, L.left_norm, L.right_norm, L.ssm_in_z, L.ssm_in_xbc,
+                                L.ssm_in_dt, L.conv_b, L.side_gate, L.side_proj, L.side_norm})
             if (t) sbytes += ggml_nbytes(t) * (uint64_t) std::max(1, times_run[(size_t) il]);  // (a layer of a repeated range is streamed once per run)
+        if (L.side_embd) sbytes += ggml_row_size(L.side_embd->type, L.side_embd->ne[0]);  // (one row of the layer's part of the side table)
         if (c.mlp == LLM_MLP_MOE) sbytes += (ggml_nbytes(L.ffn_gate_up_exps ? L.ffn_gate_up_exps : L.ffn_up_exps) + ggml_nbytes(L.ffn_down_exps)) / (uint64_t) c.n_expert * (uint64_t) c.n_top *
                                             (uint64_t) std::max(1, times_run[(size_t) il]);
         if (c.v_mix) {  // the blend factor is a scalar of the checkpoint, read once
@@ -1917,8 +2175,15 @@ static ggml_tensor * build_mixer_attention(llm_context * c, ggml_context * ctx, 
     ggml_tensor * Kcur = named(ggml_mul_mat(ctx, L.wk, cur), "Kcur", run);
     ggml_tensor * Vcur = named(ggml_mul_mat(ctx, L.wv, cur), "Vcur", run);
     ggml_tensor * gate = lc.out_gate ? named(ggml_mul_mat(ctx, L.attn_gate, cur), "attn_gate", run) : nullptr;
+    if (L.bq) Qcur = named(ggml_add(ctx, Qcur, L.bq), "Qcur_b", run);
+    if (L.bk) Kcur = named(ggml_add(ctx, Kcur, L.bk), "Kcur_b", run);
+    if (L.bv) Vcur = named(ggml_add(ctx, Vcur, L.bv), "Vcur_b", run);
     Qcur = ggml_reshape_3d(ctx, Qcur, DK, H, n_tokens);
     Kcur = ggml_reshape_3d(ctx, Kcur, DK, G, n_tokens);
+    if (lc.qk_norm) {  // every head's query and key divided by its root mean square, times a weight row shared by the heads
+        Qcur = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, Qcur, hp.rms_eps), "Qcur_rnorm", run), L.q_norm), "Qcur_normed", run);
+        Kcur = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, Kcur, hp.rms_eps), "Kcur_rnorm", run), L.k_norm), "Kcur_normed", run);
+    }
     if (lc.rot_dims > 0) {  // neighbouring pairs (2i, 2i + 1) of the leading rot_dims entries; the rest of the head passes through
         Qcur = named(ggml_rope_ext(ctx, Qcur, io.pos, nullptr, lc.rot_dims, lc.rot_half ? GGML_ROPE_TYPE_NEOX : 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Qcur_rope", run);
         Kcur = named(ggml_rope_ext(ctx, Kcur, io.pos, nullptr, lc.rot_dims, lc.rot_half ? GGML_ROPE_TYPE_NEOX : 0, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, 1.0f, 32.0f, 1.0f), "Kcur_rope", run);
@@ -1971,24 +2236,47 @@ static ggml_tensor * build_mixer_latent(llm_context * c, ggml_context * ctx, ggm
     const int64_t H = lc.n_head, DK = lc.dk, DR = lc.rot_dim, DV = lc.dv, R = lc.kv_rank, DQ = DK + DR, ROW = R + DR;
     const float mag = rope_magnitude(lc);
     (void) il;
-    ggml_tensor * Qcur = named(ggml_mul_mat(ctx, L.wq, cur), "Qcur", run);        // [DQ * H, T]: head by head [dk unrotated | dr rotated]
-    ggml_tensor * ckr = named(ggml_mul_mat(ctx, L.wdkv, cur), "kv_a", run);       // [R + DR, T]
-    ggml_tensor * lat = ggml_view_2d(ctx, ckr, R, n_tokens, ckr->nb[1], 0);
-    lat = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, lat, hp.rms_eps), "kv_a_rnorm", run), L.dkv_norm), "kv_latent", run);
-    ggml_tensor * krow = lat;
+    const int rope_mode = lc.rot_half ? GGML_ROPE_TYPE_NEOX : 0;  // pairs (i, i + dr / 2), or neighbours (2i, 2i + 1)
+    const bool own_rows = lc.kv_from < 0;                        // (else: the rows another layer's cache holds — no down projection, nothing stored)
+    // the projections of the one input follow one another: the query (or its latent), the latent of keys and values, the output gate
+    ggml_tensor * q_in = cur;
+    ggml_tensor * q_lat_pre = L.wdq ? named(ggml_mul_mat(ctx, L.wdq, cur), "q_a", run) : nullptr;
+    ggml_tensor * ckr = own_rows ? named(ggml_mul_mat(ctx, L.wdkv, cur), "kv_a", run) : nullptr;  // [R + DR, T]
+    ggml_tensor * gate = lc.out_gate ? named(ggml_mul_mat(ctx, L.attn_gate, cur), "attn_gate", run) : nullptr;
+    if (q_lat_pre) {
+        ggml_build_forward_expand(gf, q_lat_pre);
+        if (ckr) ggml_build_forward_expand(gf, ckr);
+        if (gate) ggml_build_forward_expand(gf, gate);
+        q_in = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, q_lat_pre, hp.rms_eps), "q_a_rnorm", run), L.dq_norm), "q_latent_normed", run);  // the queries' own normed latent
+    }
+    ggml_tensor * Qcur = named(ggml_mul_mat(ctx, L.wq, q_in), "Qcur", run);        // [DQ * H, T]: head by head [dk unrotated | dr rotated]
+    int cache_run = run;
+    if (!own_rows) {
+        cache_run = -1;
+        for (int r = 0; r < run; ++r)
+            if (m->runs[(size_t) r].il == lc.kv_from && m->runs[(size_t) r].pass == m->runs[(size_t) run].pass) cache_run = r;
+        LLM_ASSERT(cache_run >= 0 && c->k_l[(size_t) cache_run]);
+    }
+    ggml_tensor * k_cache = c->k_l[(size_t) cache_run];
     ggml_tensor * q_rot = nullptr;
     if (DR > 0) {
-        ggml_tensor * kr = ggml_view_3d(ctx, ckr, DR, 1, n_tokens, ckr->nb[1], ckr->nb[1], (size_t) R * sizeof(float));
-        kr = named(ggml_rope_ext(ctx, kr, io.pos, L.rope_freq, (int) DR, GGML_ROPE_TYPE_NEOX, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, mag, 32.0f, 1.0f), "k_rot", run);
-        ggml_rope_set_freq_table(kr);
-        krow = named(ggml_concat(ctx, lat, ggml_reshape_2d(ctx, kr, DR, n_tokens), 0), "kv_row", run);
         q_rot = ggml_view_3d(ctx, Qcur, DR, H, n_tokens, (size_t) DQ * sizeof(float), Qcur->nb[1], (size_t) DK * sizeof(float));
-        q_rot = named(ggml_rope_ext(ctx, q_rot, io.pos, L.rope_freq, (int) DR, GGML_ROPE_TYPE_NEOX, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, mag, 32.0f, 1.0f), "q_rot", run);
+        q_rot = named(ggml_rope_ext(ctx, q_rot, io.pos, L.rope_freq, (int) DR, rope_mode, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, mag, 32.0f, 1.0f), "q_rot", run);
         ggml_rope_set_freq_table(q_rot);
     }
-    ggml_build_forward_expand(gf, krow);
-    ggml_tensor * k_cache = c->k_l[(size_t) run];
-    ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, k_cache, krow, io.k_idxs), "kv_store", run));
+    if (own_rows) {
+        ggml_tensor * lat = ggml_view_2d(ctx, ckr, R, n_tokens, ckr->nb[1], 0);
+        lat = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, lat, hp.rms_eps), "kv_a_rnorm", run), L.dkv_norm), "kv_latent", run);
+        ggml_tensor * krow = lat;
+        if (DR > 0) {
+            ggml_tensor * kr = ggml_view_3d(ctx, ckr, DR, 1, n_tokens, ckr->nb[1], ckr->nb[1], (size_t) R * sizeof(float));
+            kr = named(ggml_rope_ext(ctx, kr, io.pos, L.rope_freq, (int) DR, rope_mode, hp.n_ctx_train, lc.rot_base, 1.0f, 0.0f, mag, 32.0f, 1.0f), "k_rot", run);
+            ggml_rope_set_freq_table(kr);
+            krow = named(ggml_concat(ctx, lat, ggml_reshape_2d(ctx, kr, DR, n_tokens), 0), "kv_row", run);
+        }
+        ggml_build_forward_expand(gf, krow);
+        ggml_build_forward_expand(gf, named(ggml_set_rows(ctx, k_cache, krow, io.k_idxs), "kv_store", run));
+    }
     // the unrotated part of every head's query, [dk, T, H] seen through strides, times W_uk,h^T -> [R, T, H]
     ggml_tensor * q_nope = ggml_view_3d(ctx, Qcur, DK, n_tokens, H, Qcur->nb[1], (size_t) DQ * sizeof(float), 0);
     ggml_tensor * q_lat = named(ggml_mul_mat(ctx, L.wuk_t, q_nope), "q_latent", run);
@@ -2002,7 +2290,9 @@ static ggml_tensor * build_mixer_latent(llm_context * c, ggml_context * ctx, ggm
     if (lc.sink) ggml_flash_attn_ext_add_sinks(att, lc.sink_learned ? L.attn_sink : ggml_view_1d(ctx, m->attn_sinks, H, 0));
     named(att, "fattn", run);
     ggml_tensor * o = named(ggml_mul_mat(ctx, L.wuv, ggml_permute(ctx, att, 0, 2, 1, 3)), "v_expand", run);  // [DV, T, H]
-    return named(ggml_cont_2d(ctx, ggml_permute(ctx, o, 0, 2, 1, 3), DV * H, n_tokens), "attn_heads", run);
+    o = named(ggml_cont_2d(ctx, ggml_permute(ctx, o, 0, 2, 1, 3), DV * H, n_tokens), "attn_heads", run);
+    if (gate) o = named(ggml_mul(ctx, o, named(ggml_unary(ctx, gate, GGML_UNARY_OP_SIGMOID), "attn_gate_sigmoid", run)), "attn_gated", run);  // one gate per value entry
+    return o;
 }
 
 // ---- mixers with state per sequence.  Each returns the mixer's output [n_embd, T] (its own output projection included).
@@ -2116,6 +2406,85 @@ static ggml_tensor * build_mixer_sigmoid_wkv(llm_context * c, ggml_context * ctx
     return named(ggml_add(ctx, named(ggml_scale(ctx, left, lc.left_scale), "mix_left", run), named(ggml_scale(ctx, right, lc.right_scale), "mix_right", run)), "mix_sum", run);
 }
 
+// state-space duality (Mamba-2): the input projection in three parts — the gate z, (x, B, C) through a short convolution with bias and SiLU, the step sizes —, the
+// recurrence per head over a state of N x dv, y times silu(z), an RMS norm over equal parts of the row, the output projection
+static ggml_tensor * build_mixer_ssd(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & lc, ggml_tensor * cur, int run, int n_tokens, seg_io & io) {
+    const int64_t H = lc.n_head, DV = lc.dv, N = lc.ssm_state, G = lc.ssm_groups, inner = H * DV, GN = G * N, NG = lc.ssm_norm_groups;
+    ggml_tensor * z = named(ggml_mul_mat(ctx, L.ssm_in_z, cur), "ssm_z", run);
+    ggml_tensor * xbc_pre = named(ggml_mul_mat(ctx, L.ssm_in_xbc, cur), "ssm_xbc_pre", run);
+    ggml_tensor * dt = named(ggml_mul_mat(ctx, L.ssm_in_dt, cur), "ssm_dt_pre", run);
+    ggml_build_forward_expand(gf, z);  // (the three products of the one input follow one another)
+    ggml_build_forward_expand(gf, xbc_pre);
+    ggml_build_forward_expand(gf, dt);
+    ggml_tensor * xbc = named(ggml_seq_conv(ctx, xbc_pre, L.conv, c->conv_state[(size_t) run], io.seq_hist, /*act=*/1), "ssm_xbc", run);
+    if (L.conv_b) ggml_seq_conv_set_bias(xbc, L.conv_b);
+    ggml_build_forward_expand(gf, xbc);  // (the state is read before it is overwritten)
+    if (lc.conv_taps > 1) ggml_build_forward_expand(gf, named(ggml_seq_conv_store(ctx, c->conv_state[(size_t) run], xbc_pre, io.seq_upd, io.seq_info, lc.conv_taps), "conv_store", run));
+    xbc = ggml_reshape_2d(ctx, xbc, xbc->ne[0], n_tokens);
+    ggml_tensor * x = ggml_view_2d(ctx, xbc, inner, n_tokens, xbc->nb[1], 0);
+    ggml_tensor * B = ggml_view_2d(ctx, xbc, GN, n_tokens, xbc->nb[1], (size_t) inner * sizeof(float));
+    ggml_tensor * C = ggml_view_2d(ctx, xbc, GN, n_tokens, xbc->nb[1], (size_t) (inner + GN) * sizeof(float));
+    ggml_tensor * y = named(ggml_seq_ssd(ctx, C, B, x, dt, L.gate_par, c->rec_state[(size_t) run], io.seq_tok, io.seq_info, (int) H, (int) G), "ssd", run);  // [DV, H, T]
+    // the gate comes before the norm
+    y = named(ggml_mul(ctx, ggml_reshape_2d(ctx, y, inner, n_tokens), named(ggml_unary(ctx, z, GGML_UNARY_OP_SILU), "ssm_z_silu", run)), "ssm_gated", run);
+    y = named(ggml_rms_norm(ctx, ggml_reshape_3d(ctx, y, inner / NG, NG, n_tokens), c->model->hp.rms_eps), "ssm_rnorm", run);
+    y = named(ggml_mul(ctx, y, ggml_reshape_2d(ctx, L.sub_norm, inner / NG, NG)), "ssm_normed", run);
+    return named(ggml_mul_mat(ctx, L.wo, ggml_reshape_2d(ctx, y, inner, n_tokens)), "attn_out", run);
+}
+
+// a gated delta rule with one decay per (head, key channel): q, k, v as one projection through short convolutions + SiLU; beta; the decay's and the output gate's
+// raw values through two small matrices each; the recurrence; per-head norm x weight x sigmoid(gate); `wo`.  Returns [n_embd, T]
+static ggml_tensor * build_mixer_delta_channel(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, ggml_tensor * wo, int H, int G, int DK, int DV, int taps,
+                                               ggml_tensor * cur, int run, int n_tokens, seg_io & io) {
+    ggml_tensor * qkv_pre = named(ggml_mul_mat(ctx, L.wqkv, cur), "delta_qkv_pre", run);
+    ggml_tensor * b_pre = named(ggml_mul_mat(ctx, L.wbeta, cur), "delta_b_pre", run);
+    ggml_tensor * a_in = named(ggml_mul_mat(ctx, L.wa1, cur), "delta_a_in", run);
+    ggml_tensor * g_in = named(ggml_mul_mat(ctx, L.wg1, cur), "delta_g_in", run);
+    ggml_build_forward_expand(gf, qkv_pre);  // (the products of the one input follow one another)
+    ggml_build_forward_expand(gf, b_pre);
+    ggml_build_forward_expand(gf, a_in);
+    ggml_build_forward_expand(gf, g_in);
+    ggml_tensor * a_pre = named(ggml_mul_mat(ctx, L.wa2, a_in), "delta_a_pre", run);  // [DK H, T]
+    ggml_tensor * gate = named(ggml_mul_mat(ctx, L.wg2, g_in), "delta_gate", run);    // [DV H, T]
+    ggml_build_forward_expand(gf, a_pre);
+    ggml_build_forward_expand(gf, gate);
+    ggml_tensor * qkv = named(ggml_seq_conv(ctx, qkv_pre, L.conv, c->conv_state[(size_t) run], io.seq_hist, /*act=*/1), "delta_qkv", run);
+    ggml_build_forward_expand(gf, qkv);  // (the state is read before it is overwritten)
+    if (taps > 1) ggml_build_forward_expand(gf, named(ggml_seq_conv_store(ctx, c->conv_state[(size_t) run], qkv_pre, io.seq_upd, io.seq_info, taps), "conv_store", run));
+    qkv = ggml_reshape_2d(ctx, qkv, qkv->ne[0], n_tokens);
+    ggml_tensor * q = ggml_view_2d(ctx, qkv, (int64_t) G * DK, n_tokens, qkv->nb[1], 0);
+    ggml_tensor * k = ggml_view_2d(ctx, qkv, (int64_t) G * DK, n_tokens, qkv->nb[1], (size_t) (G * DK) * sizeof(float));
+    ggml_tensor * v = ggml_view_2d(ctx, qkv, (int64_t) H * DV, n_tokens, qkv->nb[1], (size_t) (2 * G * DK) * sizeof(float));
+    ggml_tensor * o = named(ggml_seq_delta_channel(ctx, q, k, v, b_pre, a_pre, L.gate_par, c->rec_state[(size_t) run], io.seq_tok, io.seq_info, H, G), "delta_channel", run);
+    cur = build_head_norm_gate(ctx, o, L.sub_norm, gate, GGML_UNARY_OP_SIGMOID, c->model->hp.rms_eps, run);
+    return named(ggml_mul_mat(ctx, wo, cur), "delta_out", run);
+}
+
+// grouped-query attention (left) and the delta rule with channel decay (right) over the same input; each output is RMS-normed over the width with a weight of its own,
+// and the mixer is left_scale * left + right_scale * right
+static ggml_tensor * build_mixer_attn_delta(llm_context * c, ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & lc, ggml_tensor * cur, int il, int run,
+                                            int n_tokens, int n_kv, seg_io & io) {
+    const float eps = c->model->hp.rms_eps;
+    ggml_tensor * v_first = nullptr;
+    ggml_tensor * left = build_mixer_attention(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io, &v_first);
+    left = named(ggml_mul_mat(ctx, L.wo, left), "attn_out", run);
+    left = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, left, eps), "mix_left_rnorm", run), L.left_norm), "mix_left_normed", run);
+    ggml_build_forward_expand(gf, left);
+    ggml_tensor * right = build_mixer_delta_channel(c, ctx, gf, L, L.wo_r, lc.r_head, lc.r_head_kv, lc.r_dk, lc.r_dv, lc.conv_taps, cur, run, n_tokens, io);
+    right = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, right, eps), "mix_right_rnorm", run), L.right_norm), "mix_right_normed", run);
+    ggml_build_forward_expand(gf, right);  // (both branches first: the two SCALEs and their ADD then follow one another, which the backend runs as one blend)
+    return named(ggml_add(ctx, named(ggml_scale(ctx, left, lc.left_scale), "mix_left", run), named(ggml_scale(ctx, right, lc.right_scale), "mix_right", run)), "mix_sum", run);
+}
+
+// the per-layer token input: e = the layer's row of the side table for every token; x += rms_norm(W_proj (gelu_tanh(W_gate x) * e)) * w
+static ggml_tensor * build_token_side(ggml_context * ctx, const llm_layer & L, ggml_tensor * x, ggml_tensor * e, float eps, int run) {
+    ggml_tensor * g = named(ggml_unary(ctx, named(ggml_mul_mat(ctx, L.side_gate, x), "side_gate", run), GGML_UNARY_OP_GELU), "side_gelu", run);
+    g = named(ggml_mul(ctx, g, e), "side_gated", run);
+    ggml_tensor * y = named(ggml_mul_mat(ctx, L.side_proj, g), "side_proj", run);
+    y = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, y, eps), "side_rnorm", run), L.side_norm), "side_normed", run);
+    return named(ggml_add(ctx, x, y), "l_out_side", run);
+}
+
 // experts chosen by a soft-max over ALL experts, confined to the best groups; weights = chosen scores x scale; experts W_down (silu(W_gate h) * W_up h)
 static ggml_tensor * build_moe_grouped(ggml_context * ctx, ggml_cgraph * gf, const llm_layer & L, const llm_layer_cfg & c, ggml_tensor * cur, int il) {
     const int64_t E = cur->ne[0], T = cur->ne[1], FF = c.n_ff;
@@ -2150,7 +2519,8 @@ static ggml_tensor * build_ffn(ggml_context * ctx, ggml_cgraph * gf, const llm_l
         return named(ggml_add(ctx, named(ggml_mul_mat(ctx, L.ffn_down, cur), "ffn_down", run), L.ffn_down_b), "ffn_out", run);
     }
     cur = named(ggml_mul_mat(ctx, L.ffn_up, cur), "ffn_up", run);
-    cur = named(ggml_unary(ctx, cur, GGML_UNARY_OP_GELU_ERF), "ffn_gelu", run);
+    if (lc.ffn_relu_sq) cur = named(ggml_sqr(ctx, named(ggml_unary(ctx, cur, GGML_UNARY_OP_RELU), "ffn_relu", run)), "ffn_act", run);
+    else cur = named(ggml_unary(ctx, cur, GGML_UNARY_OP_GELU_ERF), "ffn_gelu", run);
     return named(ggml_mul_mat(ctx, L.ffn_down, cur), "ffn_out", run);
 }
 
@@ -2182,6 +2552,8 @@ static void build_layerwise(llm_context * c, ggml_context * ctx, ggml_cgraph * g
         if (lc.mixer == LLM_MIX_MLSTM) cur = build_mixer_mlstm(c, ctx, gf, L, lc, cur, run, n_tokens, io);
         else if (lc.mixer == LLM_MIX_DELTA) cur = build_mixer_delta(c, ctx, gf, L, lc, cur, run, n_tokens, io);
         else if (lc.mixer == LLM_MIX_SIGMOID_WKV) cur = build_mixer_sigmoid_wkv(c, ctx, gf, L, lc, cur, run, n_tokens, n_kv, io);
+        else if (lc.mixer == LLM_MIX_SSD) cur = build_mixer_ssd(c, ctx, gf, L, lc, cur, run, n_tokens, io);
+        else if (lc.mixer == LLM_MIX_ATTN_DELTA) cur = build_mixer_attn_delta(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io);
         else {
             cur = lc.mixer == LLM_MIX_LATENT ? build_mixer_latent(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io)
                                              : build_mixer_attention(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io, &v_first);
@@ -2193,8 +2565,14 @@ static void build_layerwise(llm_context * c, ggml_context * ctx, ggml_cgraph * g
                 inpSA = ggml_get_rows(ctx, inpSA, io.out_ids);
                 h = ggml_get_rows(ctx, h, io.out_ids);
             }
+            if (lc.two_norms && lc.mlp != LLM_MLP_NONE) h = norm_w(ctx, lc, inpSA, L.ffn_norm, eps, "ffn_norm", run);  // (the feed-forward's own norm of the same x)
             if (lc.mlp != LLM_MLP_NONE) cur = named(ggml_add(ctx, cur, build_ffn(ctx, gf, L, lc, h, il, run)), "mix_ffn", run);
             inpL = named(ggml_add(ctx, inpSA, cur), "l_out", run);
+            if (L.side_gate) {
+                ggml_tensor * e = named(ggml_get_rows(ctx, L.side_embd, io.tokens), "side_embd", run);
+                if (last && io.out_ids) e = ggml_get_rows(ctx, e, io.out_ids);
+                inpL = build_token_side(ctx, L, inpL, e, eps, run);
+            }
             continue;
         }
         if (last && io.out_ids) {
@@ -2292,7 +2670,8 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
         // layer keeps ONE row [latent | rotated key part] per token and no values beside it)
         const llm_layer_cfg * lc = layerwise ? &m->lcfg[(size_t) m->runs[(size_t) run].il] : nullptr;
         const bool latent = lc && lc->mixer == LLM_MIX_LATENT;
-        if (lc && (lc->mixer == LLM_MIX_MLSTM || lc->mixer == LLM_MIX_DELTA)) {  // (no cells: everything such a layer keeps is its sequence state)
+        if (lc && (lc->mixer == LLM_MIX_MLSTM || lc->mixer == LLM_MIX_DELTA || lc->mixer == LLM_MIX_SSD || (latent && lc->kv_from >= 0))) {
+            // (no cells: everything such a layer keeps is its sequence state — or it attends over the rows another layer's cache holds)
             c->k_l.push_back(nullptr);
             c->v_l.push_back(nullptr);
             continue;
@@ -2320,6 +2699,8 @@ extern "C" struct llm_context * llm_context_new(struct llm_model * m, ggml_backe
             int64_t conv_c = 0, rec = 0;
             if (lc.mixer == LLM_MIX_MLSTM) rec = ggml_seq_state_size(2, lc.n_head, lc.dk, lc.dv);
             else if (lc.mixer == LLM_MIX_DELTA) { conv_c = 2 * (int64_t) lc.n_head_kv * lc.dk + (int64_t) lc.n_head * lc.dv; rec = ggml_seq_state_size(1, lc.n_head, lc.dk, lc.dv); }
+            else if (lc.mixer == LLM_MIX_SSD) { conv_c = (int64_t) lc.n_head * lc.dv + 2 * (int64_t) lc.ssm_groups * lc.ssm_state; rec = ggml_seq_state_size(4, lc.n_head, lc.ssm_state, lc.dv); }
+            else if (lc.mixer == LLM_MIX_ATTN_DELTA) { conv_c = 2 * (int64_t) lc.r_head_kv * lc.r_dk + (int64_t) lc.r_head * lc.r_dv; rec = ggml_seq_state_size(3, lc.r_head, lc.r_dk, lc.r_dv); }
             else if (lc.mixer == LLM_MIX_SIGMOID_WKV) {
                 conv_c = (int64_t) (lc.n_head + lc.n_head_kv) * lc.dk + (int64_t) lc.n_head_kv * lc.dv;
                 rec = ggml_seq_state_size(0, lc.tm_heads, lc.tm_dim, lc.tm_dim);
