@@ -196,6 +196,34 @@ def rarelorn_config(z):
     return {"architecture": "Rarelorn", "layers": [mlstm, delta, par, delta], "loop": {"start": 1, "stop": 3, "times": 2}, "norm": {"eps": 1e-5}, "vocab": z["vocab"], "width": z["width"]}
 
 
+# ------------------------------------------------------------------------------------------------ --nogavik: latent attention with shared cache rows, a state-space mixer,
+# attention beside a delta rule with channel decay, a per-layer token input; beside Zigipel (dense layers, latent attention) and Rarelorn (recurrences) at equal size
+NOGAVIK_SIZES = {
+    # width, heads, kv heads, head size, latent size, rotated part, query latent, state-space heads (of 64 values: inner = 2 x width) / state / groups, taps, inner size of the
+    # decay's and the gate's matrices, side entries per layer, ff (ungated: two matrices), vocab.  Six layers: latent, state space, latent (the first layer's rows), attention +
+    # delta rule, state space, attention + delta rule — as many as the Zigipel model beside it has layer runs
+    "s": dict(width=1024, heads=8, kv=2, hd=64, rank=96, rot=32, q_rank=384, ssm_heads=32, state=128, groups=1, taps=4, low=64, side=64, ff=4128, vocab=32000),
+    "m": dict(width=2048, heads=16, kv=4, hd=128, rank=96, rot=32, q_rank=768, ssm_heads=64, state=128, groups=1, taps=4, low=128, side=128, ff=8256, vocab=32000),
+    "l": dict(width=4096, heads=32, kv=8, hd=128, rank=512, rot=64, q_rank=1536, ssm_heads=128, state=128, groups=8, taps=4, low=128, side=256, ff=14400, vocab=32000),
+}
+
+
+def nogavik_config(z):
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    H, G, D = z["heads"], z["kv"], z["hd"]
+
+    def latent(kv_from=None):
+        mx = {"heads": H, "dim": D, "rot_dim": z["rot"], "vdim": D, "kv_rank": z["rank"], "q_rank": z["q_rank"], "scale": (D + z["rot"]) ** -0.5, "rot": {"base": 1e6, "dims": z["rot"]}}
+        if kv_from is not None:
+            mx["kv_from"] = kv_from
+        return {"type": "latent_attention", "mlp": mlp, "mixer": mx}
+
+    ssm = {"type": "mamba2", "mlp": mlp, "mixer": {"heads": z["ssm_heads"], "vdim": 64, "state": z["state"], "groups": z["groups"], "norm_groups": z["groups"], "conv": z["taps"]}}
+    par = {"type": "parallel", "mlp": mlp, "mixer": {"left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5},
+                                                       "right": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": z["taps"], "rank": z["low"]}}}
+    return {"architecture": "Nogavik", "layers": [latent(), ssm, latent(0), par, ssm, par], "norm": {"eps": 1e-5}, "token_side": {"dim": z["side"]}, "vocab": z["vocab"], "width": z["width"]}
+
+
 def bench_nigozen(args):
     """Prefill and decode throughput of Nigozen models (bf16 matrices, bf16 cache, random weights) at sizes that resemble real layers, beside the
     closest existing class at equal size: llama with f16 matrices and an f16 cache (same width, layers, heads, head size, dense ff and vocabulary;
@@ -211,7 +239,7 @@ def bench_nigozen(args):
 
     be = L.Backend(0)
     n_prompt, n_dec, ub = args.prefill, max(8, min(args.steps, 64)), args.ubatch
-    if (args.zigipel or args.rarelorn) and n_prompt == 2048:
+    if (args.zigipel or args.rarelorn or args.nogavik) and n_prompt == 2048:
         # decoded positions 1984 .. 2047: a model confined to chunks of 512 / 1024 / 2048 positions then sees 449 .. 512 / 961 .. 1024 / 1985 .. 2048 cells, about as many as a
         # sliding window of the same length does (right behind a chunk's start it would see next to nothing, and the two decode steps would not compare)
         n_prompt = 1984
@@ -224,7 +252,8 @@ def bench_nigozen(args):
         prompt = rng.integers(0, n_vocab, n_prompt).tolist()
         res = {}
         best_p, best_d = None, None
-        for rep in range(2 if not (args.zigipel or args.rarelorn) else 4):  # the first pass warms up (graph capture, scratch growth); the Zigipel comparison keeps the best of the three that follow
+        best_of = bool(args.zigipel or args.rarelorn or args.nogavik)
+        for rep in range(4 if best_of else 2):  # the first pass warms up (graph capture, scratch growth); the Zigipel comparison keeps the best of the three that follow
             ctx.clear()
             be.synchronize()
             t0 = time.perf_counter()
@@ -236,8 +265,8 @@ def bench_nigozen(args):
                 assert rc == 0
             t2 = time.perf_counter()
             if rep > 0:
-                best_p = (t1 - t0) if best_p is None or not (args.zigipel or args.rarelorn) else min(best_p, t1 - t0)
-                best_d = (t2 - t1) if best_d is None or not (args.zigipel or args.rarelorn) else min(best_d, t2 - t1)
+                best_p = (t1 - t0) if best_p is None or not best_of else min(best_p, t1 - t0)
+                best_d = (t2 - t1) if best_d is None or not best_of else min(best_d, t2 - t1)
         if True:
             res = {"prefill_tok_s": round(n_prompt / best_p, 1), "decode_tok_s": round(n_dec / best_d, 1), "prefill_ms": round(best_p * 1e3, 2), "decode_ms_per_tok": round(best_d * 1e3 / n_dec, 3)}
         if os.environ.get("BENCH_NIGOZEN_CLASSES", "1") == "0":  # (a run under a profiler: its own kernel trace replaces the event-bracketed pass)
@@ -259,6 +288,27 @@ def bench_nigozen(args):
         ctx.free()
         return res
 
+    if args.nogavik:  # Nogavik beside Zigipel (as many layer runs, equal width, heads, head size, latent, vocabulary and feed-forward parameters) and Rarelorn (the recurrences)
+        out["metric"] = "nogavik_vs_zigipel_tokens_per_s"
+        out["dtype"] = "bf16 (all)"
+        be.close()
+        for name in args.nogavik.split(","):
+            z = NOGAVIK_SIZES[name]
+            zz = dict(ZIGIPEL_SIZES[name], ff=z["ff"] * 2 // 3)
+            res = {}
+            for side, cfg in (("nogavik", nogavik_config(z)), ("zigipel", zigipel_config(zz)), ("rarelorn", rarelorn_config(RARELORN_SIZES[name]))):
+                be = L.Backend(0)
+                mdl = Model(config_json=_json.dumps(cfg), seed=7, buft=be.buft, wtype=L.BF16)
+                res[side] = run(mdl, z["vocab"])
+                res[side]["weight_bytes"] = int(L.host().llm_model_total_bytes(mdl.m))
+                res[side]["stream_bytes_per_token"] = mdl.stream_bytes()
+                mdl.free()
+                be.close()
+            out["sizes"][name] = {"config": z, "nogavik": res["nogavik"], "zigipel": res["zigipel"], "rarelorn": res["rarelorn"],
+                                  "prefill_ratio": round(res["nogavik"]["prefill_tok_s"] / res["zigipel"]["prefill_tok_s"], 3),
+                                  "decode_ratio": round(res["nogavik"]["decode_tok_s"] / res["zigipel"]["decode_tok_s"], 3)}
+        print(_json.dumps(out))
+        return
     if args.rarelorn:  # Rarelorn beside Nigozen (every layer experts) with as many layers as Rarelorn has layer runs, equal width, heads, head size, vocabulary and expert parameters
         out["metric"] = "rarelorn_vs_nigozen_tokens_per_s"
         out["dtype"] = "bf16 (both)"
@@ -329,6 +379,9 @@ def main():
                     "beside Nigozen models of equal size, print one JSON line and exit; the default workload is not run")
     ap.add_argument("--rarelorn", default="", help="comma-separated sizes (s, m, l): time prefill and decode of Rarelorn models (matrix memory, gated delta rule, sigmoid attention beside "
                     "time mixing, grouped expert router, a repeated range) beside Nigozen models of equal size, print one JSON line and exit; the default workload is not run")
+    ap.add_argument("--nogavik", default="", help="comma-separated sizes (s, m, l): time prefill and decode of Nogavik models (latent attention with shared cache rows, a state-space "
+                    "mixer, attention beside a delta rule with channel decay, a per-layer token input) beside Zigipel and Rarelorn models of equal size, print one JSON line and exit; "
+                    "the default workload is not run")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
@@ -357,7 +410,7 @@ def main():
     ap.add_argument("--pmc-traffic", type=int, default=1, help="1: re-run a short decode under rocprofv3 --pmc FETCH_SIZE (own pass) for roofline.traffic")
     args = ap.parse_args()
 
-    if args.nigozen or args.zigipel or args.rarelorn:
+    if args.nigozen or args.zigipel or args.rarelorn or args.nogavik:
         bench_nigozen(args)
         return
 

@@ -171,6 +171,8 @@ _SIGS = {
     "ggml_seq_conv": (TP, [_P, TP, TP, TP, TP, _I]), "ggml_seq_conv_store": (TP, [_P, TP, TP, TP, TP, _I]),
     "ggml_seq_wkv6": (TP, [_P, TP, TP, TP, TP, TP, TP, TP, TP, TP, _I]), "ggml_seq_gated_delta": (TP, [_P, TP, TP, TP, TP, TP, TP, TP, TP, _I, _I]),
     "ggml_seq_mlstm": (TP, [_P, TP, TP, TP, TP, TP, TP, TP, TP, _I, _F]), "ggml_seq_state_size": (C.c_int64, [_I, _I, _I, _I]),
+    "ggml_seq_delta_channel": (TP, [_P, TP, TP, TP, TP, TP, TP, TP, TP, TP, _I, _I]), "ggml_seq_ssd": (TP, [_P, TP, TP, TP, TP, TP, TP, TP, TP, _I, _I]),
+    "ggml_seq_conv_set_bias": (None, [TP, TP]),
 }
 
 _host = None

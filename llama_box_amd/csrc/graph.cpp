@@ -2022,6 +2022,70 @@ static int try_fuse_head_norm_gate(exec_state & st, int i) {
     return 1;
 }
 
+// UNARY(SILU z) -> MUL(y, .) -> RMS_NORM over equal parts of the row -> MUL(w): a gate in front of a norm in parts, one launch (views between the nodes skipped).
+// Returns 1 when it ran (the nodes behind the UNARY are marked done)
+static int try_fuse_gate_norm(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * un = g->nodes[i];
+    if (un->op_params[0] != GGML_UNARY_OP_SILU || !single_use(st, un)) return 0;
+    int at[3] = {-1, -1, -1}, found = 0;
+    for (int k = i + 1; k < std::min(g->n_nodes, i + 10) && found < 3; ++k) {
+        if (st.done[k]) return 0;
+        if (is_view_op(g->nodes[k])) continue;
+        at[found++] = k;
+    }
+    if (found < 3) return 0;
+    const ggml_tensor * gm = g->nodes[at[0]], * rn = g->nodes[at[1]], * out = g->nodes[at[2]];
+    if (gm->op != GGML_OP_MUL || rn->op != GGML_OP_RMS_NORM || out->op != GGML_OP_MUL || (gm->src[0] != un && gm->src[1] != un) || gm->src[0] == gm->src[1]) return 0;
+    const ggml_tensor * y = through_views(gm->src[0] == un ? gm->src[1] : gm->src[0]), * z = un->src[0];
+    if (through_views(rn->src[0]) != gm || out->src[0] != rn || !single_use(st, gm) || !single_use(st, rn)) return 0;
+    const ggml_tensor * w = through_views(out->src[1]);
+    const int64_t D = rn->ne[0], parts = rn->ne[1], rows = rn->ne[1] * rn->ne[2] * rn->ne[3], total = D * rows;
+    if (!is_f32_contig(y) || !is_f32_contig(z) || !is_f32_contig(gm) || !is_f32_contig(rn) || !is_f32_contig(out) || !is_f32_contig(w) || !is_f32_contig(out->src[1])) return 0;
+    if (ggml_abi_nelements(y) != total || ggml_abi_nelements(z) != total || ggml_abi_nelements(gm) != total || ggml_abi_nelements(out) != total || ggml_abi_nelements(w) != D * parts) return 0;
+    // (the result may lie over y or over z entry for entry: a wave reads its whole part for the sum before it writes, and re-reads an entry right before it replaces it)
+    if (!elementwise_safe(out, y) || !elementwise_safe(out, z) || ranges_overlap(out, w)) return 0;
+    launch_gate_norm(st.c->stream, (const float *) y->data, (const float *) z->data, (const float *) w->data, (float *) out->data, D, parts, rows, ggml_abi_op_param_f32(rn, 0));
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 3;
+    for (int k = 0; k < 3; ++k) mark_done(st, at[k]);
+    return 1;
+}
+// RMS_NORM(l) -> MUL(wl), RMS_NORM(r) -> MUL(wr), SCALE, SCALE, ADD: two branches normed over the width and blended, one launch.  Returns the nodes consumed
+static int try_fuse_norm2_blend(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    if (i + 6 >= g->n_nodes) return 0;
+    for (int k = 1; k <= 6; ++k) if (st.done[i + k]) return 0;
+    const ggml_tensor * n1 = g->nodes[i], * m1 = g->nodes[i + 1], * n2 = g->nodes[i + 2], * m2 = g->nodes[i + 3], * s1 = g->nodes[i + 4], * s2 = g->nodes[i + 5], * ad = g->nodes[i + 6];
+    if (m1->op != GGML_OP_MUL || n2->op != GGML_OP_RMS_NORM || m2->op != GGML_OP_MUL || s1->op != GGML_OP_SCALE || s2->op != GGML_OP_SCALE || ad->op != GGML_OP_ADD) return 0;
+    if (m1->src[0] != n1 || m2->src[0] != n2 || s1->src[0] != m1 || s2->src[0] != m2 || ad->src[0] != s1 || ad->src[1] != s2) return 0;
+    if (ggml_abi_op_param_f32(s1, 1) != 0.0f || ggml_abi_op_param_f32(s2, 1) != 0.0f || ggml_abi_op_param_f32(n1, 0) != ggml_abi_op_param_f32(n2, 0)) return 0;
+    const ggml_tensor * l = n1->src[0], * r = n2->src[0], * wl = m1->src[1], * wr = m2->src[1];
+    for (const ggml_tensor * t : {n1, m1, n2, m2, s1, s2}) if (!single_use(st, t) || !is_f32_contig(t) || !same_shape(t, ad)) return 0;
+    if (!is_f32_contig(l) || !is_f32_contig(r) || !is_f32_contig(ad) || !same_shape(l, ad) || !same_shape(r, ad) || !is_row_of(wl, ad) || !is_row_of(wr, ad)) return 0;
+    if (!elementwise_safe(ad, l) || !elementwise_safe(ad, r) || ranges_overlap(ad, wl) || ranges_overlap(ad, wr)) return 0;
+    launch_rms_norm2_blend(st.c->stream, (const float *) l->data, (const float *) r->data, (const float *) wl->data, (const float *) wr->data, ggml_abi_op_param_f32(s1, 0),
+                           ggml_abi_op_param_f32(s2, 0), (float *) ad->data, ad->ne[0], ggml_abi_nrows(ad), ggml_abi_op_param_f32(n1, 0));
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 6;
+    return 7;
+}
+// ADD(a, b) -> ADD(x, .): the sum of two sublayers joining the stream, one launch.  Returns the nodes consumed
+static int try_fuse_add_pair(exec_state & st, int i) {
+    ggml_cgraph * g = st.g;
+    const ggml_tensor * n = g->nodes[i];
+    if (i + 1 >= g->n_nodes || st.done[i + 1]) return 0;
+    const ggml_tensor * n2 = g->nodes[i + 1], * a = n->src[0], * b = n->src[1];
+    if (n2->op != GGML_OP_ADD || (n2->src[0] != n && n2->src[1] != n) || n2->src[0] == n2->src[1] || !single_use(st, n)) return 0;
+    const ggml_tensor * x = n2->src[0] == n ? n2->src[1] : n2->src[0];
+    for (const ggml_tensor * t : {n, n2, a, b, x}) if (!is_f32_contig(t) || !same_shape(t, n2)) return 0;
+    if (!elementwise_safe(n2, a) || !elementwise_safe(n2, b) || !elementwise_safe(n2, x)) return 0;
+    launch_add3(st.c->stream, (const float *) x->data, (const float *) a->data, (const float *) b->data, (float *) n2->data, ggml_abi_nelements(n2));
+    st.c->st.kernel_launches++;
+    st.c->st.fused_nodes += 1;
+    return 2;
+}
+
 static int run_node(exec_state & st, int i);
 static bool try_fuse_geglu_bias(exec_state & st, int i) {
     ggml_cgraph * g = st.g;
@@ -2148,6 +2212,7 @@ static int run_node(exec_state & st, int i) {
 
         case GGML_OP_RMS_NORM: {
             if (fuse) { const int r = try_fuse_head_norm_gate(st, i); if (r) return r; }
+            if (fuse) { const int r = try_fuse_norm2_blend(st, i); if (r) return r; }
             // RMS_NORM -> MUL(norm, w): one kernel writing the MUL's output
             ggml_tensor * m = next(1);
             if (fuse && m && m->op == GGML_OP_MUL && single_use(st, n) && m->type == GGML_TYPE_F32 && m->nb[0] == 4) {
@@ -2184,6 +2249,19 @@ static int run_node(exec_state & st, int i) {
                     }
                     flush_deferred_splitk(st);
                     const tdesc wd = TD(w);
+                    // ... -> ADD(x, .): a normed, weighted branch joining the stream (the branch's result is read by nothing else)
+                    ggml_tensor * ad = next(2);
+                    if (ad && !st.done[i + 2] && ad->op == GGML_OP_ADD && (ad->src[0] == m || ad->src[1] == m) && ad->src[0] != ad->src[1] && single_use(st, m) && is_f32_contig(m) &&
+                        is_f32_contig(ad) && same_shape(ad, m)) {
+                        const ggml_tensor * x = ad->src[0] == m ? ad->src[1] : ad->src[0];
+                        if (is_f32_contig(x) && same_shape(x, m) && !(((uintptr_t) x->data) & 15) && elementwise_safe(ad, x) && elementwise_safe(ad, a) && !ranges_overlap(ad, w)) {
+                            timed_scope ts(c, "rms_norm_mul", (double) ggml_abi_nbytes(a) * 3);
+                            launch_rms_norm(s, TD(a), TD(ad), ggml_abi_op_param_f32(n, 0), &wd, (const float *) x->data);
+                            c->st.kernel_launches++;
+                            c->st.fused_nodes += 2;
+                            return 3;
+                        }
+                    }
                     timed_scope ts(c, "rms_norm_mul", (double) ggml_abi_nbytes(a) * 2);
                     launch_rms_norm(s, TD(a), TD(m), ggml_abi_op_param_f32(n, 0), &wd);
                     c->st.kernel_launches++;
@@ -2348,6 +2426,10 @@ static int run_node(exec_state & st, int i) {
                 const int used = try_fuse_add_chain(st, i);
                 if (used > 0) return used;
             }
+            if (fuse && row_fusions && n->op == GGML_OP_ADD) {
+                const int used = try_fuse_add_pair(st, i);
+                if (used > 0) return used;
+            }
             timed_scope ts(c, "binary", (double) ggml_abi_nbytes(n) * 3);
             launch_binary(s, n->op, TD(a), TD(b), TD(n));
             c->st.kernel_launches++;
@@ -2404,8 +2486,19 @@ static int run_node(exec_state & st, int i) {
                     }
                 }
             }
-            // SIGMOID(g) -> MUL(x, sigmoid): a gate in one pass
+            if (fuse && n->op_params[0] == GGML_UNARY_OP_SILU) { const int r = try_fuse_gate_norm(st, i); if (r) return r; }
+            // SIGMOID(g) -> MUL(x, sigmoid): a gate in one pass (likewise the tanh form of GELU and SiLU)
             ggml_tensor * gm = next(1);
+            if (fuse && (n->op_params[0] == GGML_UNARY_OP_GELU || n->op_params[0] == GGML_UNARY_OP_SILU) && gm && !st.done[i + 1] && gm->op == GGML_OP_MUL && (gm->src[0] == n || gm->src[1] == n) &&
+                gm->src[0] != gm->src[1] && single_use(st, n)) {
+                const ggml_tensor * x = gm->src[0] == n ? gm->src[1] : gm->src[0];
+                if (is_f32_contig(x) && is_f32_contig(gm) && same_shape(x, n) && same_shape(gm, n) && elementwise_safe(gm, x) && elementwise_safe(gm, a)) {
+                    launch_mul_act(s, (const float *) x->data, (const float *) a->data, (float *) gm->data, ggml_abi_nelements(gm), n->op_params[0]);
+                    c->st.kernel_launches++;
+                    c->st.fused_nodes++;
+                    return 2;
+                }
+            }
             if (fuse && n->op_params[0] == GGML_UNARY_OP_SIGMOID && gm && gm->op == GGML_OP_MUL && (gm->src[0] == n || gm->src[1] == n) && gm->src[0] != gm->src[1] && single_use(st, n)) {
                 const ggml_tensor * x = gm->src[0] == n ? gm->src[1] : gm->src[0];
                 if (is_f32_contig(x) && is_f32_contig(gm) && same_shape(x, n) && same_shape(gm, n)) {

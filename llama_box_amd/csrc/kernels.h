@@ -230,7 +230,11 @@ void launch_mmq_q80_skinny(hipStream_t s, const uint8_t * W, const uint8_t * W_p
 void launch_mmq(hipStream_t s, int type, const uint8_t * W, int64_t w_nb1, int K, int N, int M, const void * act_q8k, float * dst, int64_t dst_stride, int ksplit, float * part);
 
 // ---- element-wise / normalisation / data movement (ops.hip)
-void launch_rms_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const tdesc * mul_w /* optional fused weight */);
+void launch_rms_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const tdesc * mul_w /* optional fused weight */, const float * residual = nullptr /* optional fused ADD */);
+void launch_mul_act(hipStream_t s, const float * x, const float * g, float * d, int64_t n, int uop);     // d = x * act(g), act = GELU (tanh form) or SiLU
+void launch_add3(hipStream_t s, const float * x, const float * a, const float * b, float * d, int64_t n); // d = x + (a + b)
+void launch_gate_norm(hipStream_t s, const float * y, const float * z, const float * w, float * d, int64_t D, int64_t parts, int64_t rows, float eps);
+void launch_rms_norm2_blend(hipStream_t s, const float * l, const float * r, const float * wl, const float * wr, float a, float b, float * d, int64_t n, int64_t rows, float eps);
 void launch_layer_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const float * mul_w /* optional fused weight */, const tdesc * residual /* optional fused ADD */);
 void launch_layer_norm_twice(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const float * mul_w, const tdesc * residual, const float * w2, float eps2, const tdesc & dst2);  // ... and dst2 = LN(dst) * w2
 void launch_topk_softmax(hipStream_t s, const tdesc & logits /* [n, T] */, const tdesc & ids /* [n, T] i32: the descending permutation */, const tdesc & wts /* [k, T] */, int k);  // k <= 256

@@ -60,7 +60,8 @@ __device__ __forceinline__ void q80_panel_store(const float r0, const float r1, 
 // Q80P (round 6): the row leaves as Q8_0 blocks in panel order instead of f32 — every reader is a Q8_0 mat-mul of 9 .. 128 columns (graph.cpp: q80_panel_consumers_only);
 // the vector path only (the launcher checks), same arithmetic as the two kernels it replaces
 template <bool Q80P>
-__global__ void __launch_bounds__(256) k_rms_norm(const tdesc a, const tdesc d, const float eps, const float * __restrict__ w, char * __restrict__ q80 = nullptr) {
+__global__ void __launch_bounds__(256) k_rms_norm(const tdesc a, const tdesc d, const float eps, const float * __restrict__ w, char * __restrict__ q80 = nullptr,
+                                                  const float * res = nullptr /* rows like d's, contiguous: added to the normed, weighted row (the ADD behind the MUL) */) {
     __shared__ double sh[4];
     const int64_t row = blockIdx.x;
     const int64_t i1 = row % a.ne[1], i2 = (row / a.ne[1]) % a.ne[2], i3 = row / (a.ne[1] * a.ne[2]);
@@ -108,6 +109,7 @@ __global__ void __launch_bounds__(256) k_rms_norm(const tdesc a, const tdesc d, 
                     float4 r;
                     r.x = v[u].x * scale; r.y = v[u].y * scale; r.z = v[u].z * scale; r.w = v[u].w * scale;
                     if (w) { r.x = r.x * g[u].x; r.y = r.y * g[u].y; r.z = r.z * g[u].z; r.w = r.w * g[u].w; }
+                    if (res) { const float4 e = ((const float4 *) (res + row * n))[i]; r.x = r.x + e.x; r.y = r.y + e.y; r.z = r.z + e.z; r.w = r.w + e.w; }
                     if constexpr (Q80P) q80_panel_store(r.x, r.y, r.z, r.w, (int) (i & 7), row, i >> 3, n >> 5, q80);
                     else y4[i] = r;
                 }
@@ -117,13 +119,14 @@ __global__ void __launch_bounds__(256) k_rms_norm(const tdesc a, const tdesc d, 
         for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
             float v = x[i] * scale;
             if (w) v = v * w[i];
+            if (res) v = v + res[row * n + i];
             y[i] = v;
         }
     }
 }
-void launch_rms_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const tdesc * mul_w) {
+void launch_rms_norm(hipStream_t s, const tdesc & src, const tdesc & dst, float eps, const tdesc * mul_w, const float * residual) {
     const int64_t rows = src.ne[1] * src.ne[2] * src.ne[3];
-    hipLaunchKernelGGL(k_rms_norm<false>, dim3((unsigned) rows), dim3(256), 0, s, src, dst, eps, mul_w ? (const float *) mul_w->data : nullptr, (char *) nullptr);
+    hipLaunchKernelGGL(k_rms_norm<false>, dim3((unsigned) rows), dim3(256), 0, s, src, dst, eps, mul_w ? (const float *) mul_w->data : nullptr, (char *) nullptr, residual);
 }
 bool rms_norm_q80_panel_ok(const tdesc & src, const float * w) {  // the kernel's vector path, whole Q8_0 blocks
     return (src.ne[0] % 32) == 0 && src.nb[0] == 4 && ((((uintptr_t) src.data) | ((uintptr_t) w) | (uintptr_t) src.nb[1] | (uintptr_t) src.nb[2] | (uintptr_t) src.nb[3]) & 15) == 0;
@@ -480,6 +483,84 @@ __global__ void __launch_bounds__(256) k_mul_sigmoid(const float * __restrict__ 
 void launch_mul_sigmoid(hipStream_t s, const float * x, const float * g, float * d, int64_t n) {
     if (n == 0) return;
     hipLaunchKernelGGL(k_mul_sigmoid, dim3((unsigned) std::min<int64_t>((n + 255) / 256, 2048)), dim3(256), 0, s, x, g, d, n);
+}
+// x * act(g) with act = the tanh form of GELU or SiLU (UNARY -> MUL; k_unary's formulas), and x + (a + b) (two ADDs)
+__global__ void __launch_bounds__(256) k_mul_act(const float * __restrict__ x, const float * __restrict__ g, float * __restrict__ d, const int64_t n, const int uop) {
+    for (int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t) gridDim.x * blockDim.x) {
+        const float v = g[i];
+        const float r = uop == GGML_UNARY_OP_SILU ? silu_f(v) : 0.5f * v * (1.0f + tanhf(0.79788456080286535588f * (v + 0.044715f * v * v * v)));
+        d[i] = x[i] * r;
+    }
+}
+void launch_mul_act(hipStream_t s, const float * x, const float * g, float * d, int64_t n, int uop) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(k_mul_act, dim3((unsigned) std::min<int64_t>((n + 255) / 256, 2048)), dim3(256), 0, s, x, g, d, n, uop);
+}
+__global__ void __launch_bounds__(256) k_add3(const float * __restrict__ x, const float * __restrict__ a, const float * __restrict__ b, float * __restrict__ d, const int64_t n) {
+    for (int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t) gridDim.x * blockDim.x) {
+        const float t = a[i] + b[i];
+        d[i] = x[i] + t;
+    }
+}
+void launch_add3(hipStream_t s, const float * x, const float * a, const float * b, float * d, int64_t n) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(k_add3, dim3((unsigned) std::min<int64_t>((n + 255) / 256, 2048)), dim3(256), 0, s, x, a, b, d, n);
+}
+// a gate in FRONT of a norm over equal parts of a row: t = y * silu(z); every part of D entries divided by its root mean square; times w (one entry per entry of the
+// row) — UNARY(SILU) -> MUL -> RMS_NORM -> MUL.  A wave per (part, token); the sum of squares in f64 as in k_rms_norm
+__global__ void __launch_bounds__(256) k_gate_norm(const float * y, const float * z, const float * __restrict__ w, float * d, const int64_t D, const int64_t parts, const int64_t rows,
+                                                   const float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t) blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int64_t p = row % parts;
+    const float * yr = y + row * D, * zr = z + row * D;
+    double s = 0.0;
+    for (int64_t i = lane; i < D; i += 64) { const float t = yr[i] * silu_f(zr[i]); s += (double) (t * t); }
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    const float mean = (float) (s / (double) D);
+    const float scale = 1.0f / sqrtf(mean + eps);
+    const float * __restrict__ wr = w + p * D;
+    float * out = d + row * D;
+    for (int64_t i = lane; i < D; i += 64) {
+        const float t = yr[i] * silu_f(zr[i]);
+        const float v = t * scale;
+        out[i] = v * wr[i];
+    }
+}
+void launch_gate_norm(hipStream_t s, const float * y, const float * z, const float * w, float * d, int64_t D, int64_t parts, int64_t rows, float eps) {
+    if (rows == 0 || D == 0) return;
+    hipLaunchKernelGGL(k_gate_norm, dim3((unsigned) ((rows + 3) / 4)), dim3(256), 0, s, y, z, w, d, D, parts, rows, eps);
+}
+// two rows normed and blended: d = a * (rms_norm(l) * wl) + b * (rms_norm(r) * wr) — RMS_NORM -> MUL, RMS_NORM -> MUL, SCALE, SCALE, ADD.  A workgroup per row; the sums
+// are taken as k_rms_norm takes them on its element-wise path
+__global__ void __launch_bounds__(256) k_rms_norm2_blend(const float * l, const float * r, const float * __restrict__ wl, const float * __restrict__ wr, const float a, const float b,
+                                                         float * d, const int64_t n, const float eps) {
+    __shared__ double sh[4];
+    const int64_t row = blockIdx.x;
+    const float * x = l + row * n, * y = r + row * n;
+    double s = 0.0, u = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = x[i], q = y[i];
+        s += (double) (v * v);
+        u += (double) (q * q);
+    }
+    s = block_sum_d(s, sh);
+    __syncthreads();
+    u = block_sum_d(u, sh);
+    const float sl = 1.0f / sqrtf((float) (s / (double) n) + eps), sr = 1.0f / sqrtf((float) (u / (double) n) + eps);
+    float * out = d + row * n;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = x[i] * sl, q = y[i] * sr;
+        v = v * wl[i];
+        q = q * wr[i];
+        const float pa = v * a, pb = q * b;
+        out[i] = pa + pb;
+    }
+}
+void launch_rms_norm2_blend(hipStream_t s, const float * l, const float * r, const float * wl, const float * wr, float a, float b, float * d, int64_t n, int64_t rows, float eps) {
+    if (rows == 0 || n == 0) return;
+    hipLaunchKernelGGL(k_rms_norm2_blend, dim3((unsigned) rows), dim3(256), 0, s, l, r, wl, wr, a, b, d, n, eps);
 }
 __global__ void __launch_bounds__(256) k_weighted_rows_sum(const tdesc rows, const tdesc w, const tdesc d) {
     const int64_t t = blockIdx.x, n_used = rows.ne[1];

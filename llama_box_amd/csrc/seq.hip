@@ -187,7 +187,7 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
 #pragma unroll
         for (int i = 0; i < SEQ_NV; ++i) {
             if (lane + 64 * i < TB * per_tok)
-                dstb[lane + 64 * i] = (HAS_W && f >= off_w && f < off_v) ? (KIND == SEQ_WKV6 ? expf(-expf(pre[i])) : expf(-a_exp * seq_softplus(pre[i]))) : pre[i];
+                dstb[lane + 64 * i] = (KIND == SEQ_WKV6 && f >= off_w && f < off_v) ? expf(-expf(pre[i])) : pre[i];
             f += 64;
             f = f >= per_tok ? f - per_tok : f;
         }
@@ -206,6 +206,16 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
             *gp = y;
         }
     };
+    // channel decay: the parked raw values (projection + offset) of a block's n_tok tokens become exp(-e^A softplus(.)) — the lanes walk over the DK real entries of
+    // every token only, so the softplus and the two exponentials are paid once per entry (not once per staged float)
+    auto finish_decay = [&](float * dstb, const int n_tok) {
+        if (KIND == SEQ_DELTA_CH)
+            for (int idx = lane; idx < n_tok * DK; idx += 64) {
+                const int u = idx / DK, fe = idx - u * DK;
+                float * wp = dstb + u * per_tok + off_w + fe;
+                *wp = expf(-a_exp * seq_softplus(*wp));
+            }
+    };
     float pre[SEQ_NV];
     if (lane < SEQ_MAX_TB) {
         rows_of[0][lane] = lane < count ? A.tok[begin + lane] : 0;
@@ -216,6 +226,7 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
     park(blk[0], pre);
     __syncthreads();
     finish_gates(blk[0]);
+    finish_decay(blk[0], min(TB, count));
     __syncthreads();
     for (int b0 = 0, b = 0; b0 < count; b0 += TB, ++b) {
         const int n_here = min(TB, count - b0), n_next = min(TB, count - b0 - TB);
@@ -346,6 +357,7 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
             if (lane < TB) rows_of[b & 1][lane] = row_after;
             __syncthreads();
             finish_gates(blk[(b + 1) & 1]);
+            finish_decay(blk[(b + 1) & 1], n_next);
         }
         __syncthreads();
     }

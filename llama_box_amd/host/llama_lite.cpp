@@ -2468,11 +2468,11 @@ static ggml_tensor * build_mixer_attn_delta(llm_context * c, ggml_context * ctx,
     ggml_tensor * v_first = nullptr;
     ggml_tensor * left = build_mixer_attention(c, ctx, gf, L, lc, cur, il, run, n_tokens, n_kv, io, &v_first);
     left = named(ggml_mul_mat(ctx, L.wo, left), "attn_out", run);
-    left = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, left, eps), "mix_left_rnorm", run), L.left_norm), "mix_left_normed", run);
     ggml_build_forward_expand(gf, left);
     ggml_tensor * right = build_mixer_delta_channel(c, ctx, gf, L, L.wo_r, lc.r_head, lc.r_head_kv, lc.r_dk, lc.r_dv, lc.conv_taps, cur, run, n_tokens, io);
+    ggml_build_forward_expand(gf, right);  // (both branches first: the two norms, the two SCALEs and their ADD then follow one another, which the backend runs as one launch)
+    left = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, left, eps), "mix_left_rnorm", run), L.left_norm), "mix_left_normed", run);
     right = named(ggml_mul(ctx, named(ggml_rms_norm(ctx, right, eps), "mix_right_rnorm", run), L.right_norm), "mix_right_normed", run);
-    ggml_build_forward_expand(gf, right);  // (both branches first: the two SCALEs and their ADD then follow one another, which the backend runs as one blend)
     return named(ggml_add(ctx, named(ggml_scale(ctx, left, lc.left_scale), "mix_left", run), named(ggml_scale(ctx, right, lc.right_scale), "mix_right", run)), "mix_sum", run);
 }
 
@@ -2571,6 +2571,7 @@ static void build_layerwise(llm_context * c, ggml_context * ctx, ggml_cgraph * g
             if (L.side_gate) {
                 ggml_tensor * e = named(ggml_get_rows(ctx, L.side_embd, io.tokens), "side_embd", run);
                 if (last && io.out_ids) e = ggml_get_rows(ctx, e, io.out_ids);
+                ggml_build_forward_expand(gf, e);  // (the rows first: the gate's activation and its product with them then follow one another)
                 inpL = build_token_side(ctx, L, inpL, e, eps, run);
             }
             continue;

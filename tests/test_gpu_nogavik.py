@@ -1,0 +1,625 @@
+"""GPU tests of the Nogavik model class: the engine (llama_lite over the MI355X backend) against the plain numpy reference of
+tests/nogavik_ref.py, on small models with their own sizes and random weights.
+
+f32 serving is the sharp instrument: with 32-bit arithmetic end to end a key wrongly seen or hidden, a rotation pair taken the wrong way, a
+convolution tap from the wrong token, a lost state or cache rows read from the wrong layer moves a logit row by 1e-3 of its spread and more,
+ten times the gate (1e-4).  bf16 serving is gated at its rounding level.  Where random data could hide a fault (one key far back among
+hundreds, the first tokens of a long sequence, a constant of a recurrence) a test shows that the data discriminate: the same rows are far
+from the reference computed with the neighbouring rule."""
+import copy
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import harness as T
+import llama_box_amd as L
+import nogavik_ref as R
+from llama_box_amd.trace import TraceSession
+
+pytestmark = pytest.mark.gpu
+
+F32_GATE, BF16_GATE = 1e-4, 5e-2
+
+
+def row_err(got, ref):
+    """per row: rms of the difference (means removed) over the rms of the reference row (mean removed)"""
+    d = got - ref
+    d = d - d.mean(axis=-1, keepdims=True)
+    r = ref - ref.mean(axis=-1, keepdims=True)
+    return np.sqrt((d * d).mean(axis=-1)) / np.sqrt((r * r).mean(axis=-1))
+
+
+def within(e, gate, dtype):
+    """f32: every row within the gate.  bf16: the design norms several small vectors (the side input's few entries, a branch's output at the first positions); where such
+    a vector comes out of cancellation its norm magnifies bf16's rounding at that one position, so 19 rows in 20 are within the gate and none is beyond three times it"""
+    e = np.asarray(e)
+    if dtype == "f32":
+        return bool(e.max() <= gate)
+    return bool(np.quantile(e, 0.95) <= gate and e.max() <= 3 * gate)
+
+
+def toks(n, vocab, seed):
+    return np.random.default_rng(seed).integers(0, vocab, n).tolist()
+
+
+def cfg_a():
+    # every mixer; a latent layer that reads the first layer's cache rows; 3 query heads per key head; key size != value size; taps 3 and 4; two groups of (B, C);
+    # a norm in two parts; a layer without feed-forward
+    return R.make_config(64, 97, [
+        R.latent_layer(heads=4, dim=12, rot_dim=8, vdim=20, kv_rank=24, q_rank=16, scale=0.21, mlp=R.dense(48), base=100.0),
+        R.state_space_layer(heads=4, vdim=12, state=10, groups=2, norm_groups=2, conv=3, mlp=R.dense(40)),
+        R.latent_layer(heads=2, dim=20, rot_dim=8, vdim=12, kv_rank=24, q_rank=12, scale=0.17, mlp=None, base=100.0, kv_from=0),
+        R.parallel_layer(heads=6, kv_heads=2, dim=16, vdim=24, scale=0.2, r_heads=4, r_kv_heads=2, r_dim=12, r_vdim=20, conv=4, mlp=R.dense(56), rank=6),
+    ], side_dim=10, eps=3e-5)
+
+
+def cfg_b():
+    # rows that are no multiple of 8 (width 52); the parallel mixer first; one head everywhere; a state beyond 128 entries; one tap (no history); key rows that are no
+    # multiple of 4; no rotated part at all
+    return R.make_config(52, 50, [
+        R.parallel_layer(heads=1, kv_heads=1, dim=12, vdim=20, scale=0.3, r_heads=1, r_kv_heads=1, r_dim=14, r_vdim=10, conv=1, mlp=R.dense(12), rank=3),
+        R.state_space_layer(heads=1, vdim=6, state=136, groups=1, norm_groups=1, conv=2, mlp=None),
+        R.latent_layer(heads=3, dim=10, rot_dim=0, vdim=6, kv_rank=9, q_rank=7, scale=0.3, mlp=R.dense(20)),
+    ], side_dim=3, eps=1e-6)
+
+
+def cfg_c():
+    # no attention anywhere (no cells are read, no positions); no side input; norm parts equal to the heads
+    return R.make_config(48, 257, [
+        R.state_space_layer(heads=4, vdim=8, state=16, groups=4, norm_groups=4, conv=4, mlp=R.dense(24)),
+        R.state_space_layer(heads=6, vdim=4, state=5, groups=3, norm_groups=1, conv=1, mlp=R.dense(24)),
+    ], side_dim=0, eps=1e-5)
+
+
+def cfg_d():
+    # wide heads (a value row beyond 128), a latent row of 136 + 24; two layers reading one earlier layer's rows; every entry of the rotated part is the whole key's
+    # rotated share; a large rotation base
+    return R.make_config(96, 120, [
+        R.latent_layer(heads=3, dim=40, rot_dim=24, vdim=136, kv_rank=136, q_rank=40, scale=0.12, mlp=R.dense(32), base=20000.0),
+        R.latent_layer(heads=5, dim=8, rot_dim=24, vdim=16, kv_rank=136, q_rank=24, scale=0.2, mlp=None, base=20000.0, kv_from=0),
+        R.parallel_layer(heads=4, kv_heads=4, dim=40, vdim=136, scale=0.12, r_heads=3, r_kv_heads=3, r_dim=32, r_vdim=24, conv=3, mlp=R.dense(32), rank=8),
+        R.latent_layer(heads=2, dim=16, rot_dim=24, vdim=8, kv_rank=136, q_rank=8, scale=0.25, mlp=R.dense(16), base=20000.0, kv_from=0),
+    ], side_dim=24, eps=1e-6)
+
+
+CONFIGS = {"a": cfg_a, "b": cfg_b, "c": cfg_c, "d": cfg_d}
+
+
+class Served:
+    def __init__(self, backend, tmp_path, cfg, seed, dtype, max_tokens=512, n_ubatch=64, W=None):
+        self.cfg, self.W = cfg, W if W is not None else R.random_weights(cfg, seed)
+        R.save_model(cfg, self.W, str(tmp_path))
+        self.s = TraceSession(str(tmp_path), "float32" if dtype == "f32" else "bfloat16", max_tokens=max_tokens, n_ubatch=n_ubatch, backend=backend)
+        self.gate = F32_GATE if dtype == "f32" else BF16_GATE
+
+    def ref(self, tokens):
+        return R.forward(self.cfg, self.W, tokens)
+
+    def feed(self, rid, tokens, end=False):
+        return self.s.step([{"id": rid, "tokens": list(tokens), "want": list(range(len(tokens)))}], [rid] if end else [])
+
+    def free(self):
+        self.s.close()
+
+
+# ------------------------------------------------------------------------------------------------ whole models through the engine
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("which", ["a", "b", "c", "d"])
+def test_whole_prompt(backend, tmp_path, plog, which, dtype):
+    s = Served(backend, tmp_path, CONFIGS[which](), 11, dtype)
+    t = toks(150, s.cfg["vocab"], 5)  # three micro-batches of 64 / 64 / 22 tokens; every position's logits
+    e = row_err(s.feed("w", t, end=True), s.ref(t))
+    plog(f"nogavik whole prompt cfg {which} {dtype}: max row error {e.max():.3e}, median {np.median(e):.3e}")
+    assert within(e, s.gate, dtype), (int(np.argmax(e)), float(e.max()))
+    s.free()
+
+
+def one_layer(kind, **kw):
+    if kind == "latent":
+        d = dict(heads=3, dim=12, rot_dim=8, vdim=20, kv_rank=16, q_rank=12, scale=0.2, mlp=None, base=100.0)
+        d.update(kw)
+        return R.latent_layer(**d)
+    if kind == "ssd":
+        d = dict(heads=4, vdim=8, state=12, groups=2, norm_groups=1, conv=3, mlp=None)
+        d.update(kw)
+        return R.state_space_layer(**d)
+    d = dict(heads=4, kv_heads=2, dim=16, vdim=12, scale=0.25, r_heads=4, r_kv_heads=2, r_dim=12, r_vdim=8, conv=3, mlp=None, rank=4)
+    d.update(kw)
+    return R.parallel_layer(**d)
+
+
+@pytest.mark.parametrize("case", ["latent", "latent_no_rotation", "latent_shared_rows", "ssd", "ssd_one_tap", "ssd_norm_parts", "attention_alone", "delta_alone", "parallel",
+                                  "feed_forward", "no_side_input", "side_of_one", "equal_sizes"])
+def test_one_mechanism_at_a_time(backend, tmp_path, case):
+    """small models with one mixer and nothing else (or one more part behind a fixed mixer), so that a fault has one place to be"""
+    side, zero = 6, None
+    if case == "latent":
+        layers = [one_layer("latent")]
+    elif case == "latent_no_rotation":
+        layers = [one_layer("latent", rot_dim=0)]
+    elif case == "latent_shared_rows":
+        layers = [one_layer("latent"), one_layer("latent", heads=2, dim=8, vdim=4, q_rank=5, kv_from=0)]
+    elif case == "ssd":
+        layers = [one_layer("ssd")]
+    elif case == "ssd_one_tap":
+        layers = [one_layer("ssd", conv=1, groups=1)]
+    elif case == "ssd_norm_parts":
+        layers = [one_layer("ssd", norm_groups=4, groups=4)]
+    elif case == "attention_alone":
+        layers, zero = [one_layer("parallel")], "l0.mix.right.out"
+    elif case == "delta_alone":
+        layers, zero = [one_layer("parallel")], "l0.mix.left.out"
+    elif case == "parallel":
+        layers = [one_layer("parallel")]
+    elif case == "feed_forward":
+        layers = [one_layer("ssd", mlp=R.dense(24))]
+    elif case == "no_side_input":
+        layers, side = [one_layer("latent", mlp=R.dense(24))], 0
+    elif case == "side_of_one":  # (one entry: the normed side input is the projection's column with the sign of the gated entry)
+        layers, side = [one_layer("ssd"), one_layer("latent")], 1
+    else:  # sizes that coincide: one head per key head, key size = value size = state, rank = side size
+        layers = [one_layer("parallel", heads=2, kv_heads=2, dim=8, vdim=8, r_heads=2, r_kv_heads=2, r_dim=8, r_vdim=8, rank=8), one_layer("ssd", heads=2, vdim=8, state=8, groups=2, norm_groups=2)]
+        side = 8
+    cfg = R.make_config(48, 40, layers, side_dim=side)
+    W = R.random_weights(cfg, 21)
+    if zero:
+        W[zero] = W[zero] * 0.0
+    s = Served(backend, tmp_path, cfg, 0, "f32", W=W)
+    t = toks(40, 40, 3)
+    e = row_err(s.feed("w", t, end=True), s.ref(t))
+    assert e.max() <= F32_GATE, (int(np.argmax(e)), float(e.max()))
+    s.free()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("which", ["a", "d"])
+def test_prefill_against_token_by_token(backend, tmp_path, which, dtype):
+    s = Served(backend, tmp_path, CONFIGS[which](), 12, dtype)
+    t = toks(45, s.cfg["vocab"], 6)
+    # the first tokens of a sequence one at a time: position 0 reads no state, no convolution history and an empty cache
+    rows = np.concatenate([s.feed("x", [tok]) for tok in t])
+    ref = s.ref(t)
+    assert within(row_err(rows, ref), s.gate, dtype)
+    whole = s.feed("y", t, end=True)
+    assert within(row_err(whole, rows.astype(np.float64)), 2e-5 if dtype == "f32" else s.gate, dtype)
+    s.free()
+
+
+@pytest.mark.parametrize("which", ["a", "b", "c", "d"])
+def test_portions_of_every_size(backend, tmp_path, which):
+    s = Served(backend, tmp_path, CONFIGS[which](), 13, "f32")
+    t = toks(131, s.cfg["vocab"], 7)
+    cuts = [2, 3, 2, 7, 1, 16, 5, 2, 64, 2, 9, 18]  # down to two tokens; cuts fall inside the reach of the convolutions (fewer tokens than taps) and inside blocks of cells
+    assert sum(cuts) == len(t)
+    at, rows = 0, []
+    for n in cuts:
+        rows.append(s.feed("x", t[at:at + n]))
+        at += n
+    e = row_err(np.concatenate(rows), s.ref(t))
+    assert e.max() <= s.gate, (int(np.argmax(e)), float(e.max()))
+    s.free()
+
+
+def test_long_decoding(backend, tmp_path):
+    s = Served(backend, tmp_path, cfg_a(), 14, "f32", max_tokens=512)
+    t = toks(330, s.cfg["vocab"], 8)  # 3 prompt tokens, then single steps: the used part of the cache grows past 256 cells, every state is carried 327 times
+    rows = [s.feed("x", t[:3])] + [s.feed("x", [tok]) for tok in t[3:]]
+    e = row_err(np.concatenate(rows), s.ref(t))
+    assert e.max() <= s.gate, (int(np.argmax(e)), float(e.max()))
+    s.free()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_unequal_requests_in_mixed_batches_with_cells_and_slots_used_again(backend, tmp_path, dtype):
+    cfg = cfg_a()
+    reqs = {name: toks(n, cfg["vocab"], 20 + i) for i, (name, n) in enumerate([("p", 190), ("q", 33), ("r", 1), ("s", 240), ("t", 57), ("u", 175), ("v", 2)])}
+    # 256 + 4 x 64 cells for 698 tokens in total: the cells of ended requests are handed out again, as are the four sequence slots with their states
+    sv = Served(backend, tmp_path, cfg, 15, dtype, max_tokens=256, n_ubatch=64)
+    fed = {k: 0 for k in reqs}
+    got = {k: [] for k in reqs}
+    plan = [  # (request, tokens) per step: portions beside single tokens, requests left out of steps, ends in between
+        [("p", 40), ("q", 2)], [("p", 1), ("q", 30), ("r", 1)], [("p", 1), ("q", 1), ("s", 64), ("v", 2)], [("p", 148), ("s", 3)], [("s", 173)],
+        [("t", 20), ("u", 2)], [("t", 1), ("u", 170)], [("u", 1), ("t", 36)], [("u", 2)],
+    ]
+    for step in plan:
+        entries, ends = [], []
+        for name, n in step:
+            a = fed[name]
+            entries.append({"id": name, "tokens": reqs[name][a:a + n], "want": list(range(n))})
+            fed[name] = a + n
+            if fed[name] == len(reqs[name]):
+                ends.append(name)
+        rows = sv.s.step(entries, ends)
+        at = 0
+        for name, n in step:
+            got[name].append(rows[at:at + n])
+            at += n
+    for k in reqs:
+        assert fed[k] == len(reqs[k])
+        e = row_err(np.concatenate(got[k]), sv.ref(reqs[k]))
+        assert within(e, sv.gate, dtype) or (len(e) < 20 and e.max() <= 3 * sv.gate), (k, int(np.argmax(e)), float(e.max()))
+    sv.free()
+
+
+def test_batched_requests_give_what_each_gives_alone(backend, tmp_path):
+    """the same three requests alone and side by side in one batch: the rows agree to rounding (a batch changes which mat-mul tiling runs, nothing else)"""
+    cfg = cfg_d()
+    reqs = [toks(n, cfg["vocab"], 70 + i) for i, n in enumerate((37, 5, 64))]
+    s = Served(backend, tmp_path, cfg, 19, "f32")
+    alone = [s.feed("a%d" % i, r, end=True) for i, r in enumerate(reqs)]
+    rows = s.s.step([{"id": "b%d" % i, "tokens": r, "want": list(range(len(r)))} for i, r in enumerate(reqs)], ["b0", "b1", "b2"])
+    at = 0
+    for i, r in enumerate(reqs):
+        assert row_err(rows[at:at + len(r)], alone[i].astype(np.float64)).max() <= 2e-5
+        at += len(r)
+    s.free()
+
+
+def test_a_slot_used_again_starts_from_nothing(backend, tmp_path):
+    """a request that takes over the slot (recurrence matrices, convolution history) and the cells of an ended one gives what it gives alone"""
+    s = Served(backend, tmp_path, cfg_a(), 16, "f32", max_tokens=64)
+    a, b = toks(50, s.cfg["vocab"], 1), toks(60, s.cfg["vocab"], 2)
+    s.feed("a", a, end=True)
+    rows = np.concatenate([s.feed("b", b[:1]), s.feed("b", b[1:7]), s.feed("b", b[7:], end=True)])
+    assert row_err(rows, s.ref(b)).max() <= F32_GATE
+    s.free()
+
+
+def test_greedy_generation_through_the_engine(backend, tmp_path, H):
+    s = Served(backend, tmp_path, cfg_a(), 17, "f32")
+    prompt = toks(9, s.cfg["vocab"], 9)
+    s.s.step([{"id": "g", "tokens": prompt, "want": [len(prompt) - 1]}], [])
+    seq = list(prompt)
+    for _ in range(24):
+        tok = H.llm_sample_greedy(s.s.ctx, -1)  # the engine's own sampler on the engine's own logits
+        ref_row = s.ref(seq)[-1]
+        top2 = np.sort(ref_row)[-2:]
+        if top2[1] - top2[0] > 1e-3 * np.abs(ref_row).max():
+            assert tok == int(np.argmax(ref_row))
+        else:
+            tok = int(np.argmax(ref_row))
+        seq.append(tok)
+        s.s.step([{"id": "g", "tokens": [tok], "want": [0]}], [])
+    s.free()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_fused_steps_equal_the_unfused_nodes(backend, tmp_path, dtype):
+    """the fused launches (norm with weight, the latent cache row and the query row with neighbouring rotation pairs, sigmoid gates, squared ReLU, the per-head norm with
+    gate, the blend of the two branches, sibling mat-vecs): bit for bit what the graph's own nodes give, for a prompt portion and for single tokens"""
+    cfg = cfg_a()
+    t = toks(90, cfg["vocab"], 41)
+    rows, launches = {}, {}
+    for fusion in (1, 0):
+        backend.set_option("fusion", fusion)
+        s = Served(backend, tmp_path / str(fusion), cfg, 18, dtype)
+        before = backend.stat("kernel_launches")
+        rows[fusion] = np.concatenate([s.feed("x", t[:70])] + [s.feed("x", [tok]) for tok in t[70:]])
+        launches[fusion] = backend.stat("kernel_launches") - before
+        s.free()
+    backend.set_option("fusion", 1)
+    assert np.array_equal(rows[0], rows[1])
+    assert launches[1] < 0.9 * launches[0], launches
+
+
+# ------------------------------------------------------------------------------------------------ the data must show a rule that is one off
+@pytest.mark.parametrize("how", ["prompt", "decoded"])
+def test_rotation_scale_gate_and_shared_rows_show(backend, tmp_path, how):
+    """two latent layers, the second reading the first one's rows: the engine's rows match the reference with exactly these rules and are far from the reference with
+    rotate-half pairs, another base, another scale, the second layer's rows taken from a projection of its own, or no output gate"""
+    cfg = R.make_config(48, 40, [one_layer("latent", rot_dim=12), one_layer("latent", rot_dim=12, heads=2, q_rank=6, kv_from=0)], side_dim=4)
+    W = R.random_weights(cfg, 31)
+    for name in list(W):
+        if name.endswith("mix.uq"):
+            W[name] = R.bf16_round(W[name] * 3.0)  # sharper scores: one key that comes or goes is seen
+    s = Served(backend, tmp_path, cfg, 0, "f32", W=W)
+    t = toks(60, 40, 4)
+    rows = s.feed("w", t, end=True) if how == "prompt" else np.concatenate([s.feed("w", t[:5])] + [s.feed("w", [x]) for x in t[5:]])
+    assert row_err(rows, R.forward(cfg, W, t)).max() <= F32_GATE
+    tail = slice(10, 60)
+
+    def far_from(ref_rows):
+        return row_err(rows[tail], ref_rows[tail]).max() > 20 * F32_GATE
+
+    for key, val in (("scale", 0.21), ("base", 90.0)):
+        c2 = copy.deepcopy(cfg)
+        for Lc in c2["layers"]:
+            if key == "base":
+                Lc["mixer"]["rot"]["base"] = val
+            else:
+                Lc["mixer"][key] = val
+        assert far_from(R.forward(c2, W, t)), key
+    saved = R.rotate_pairs
+    try:
+        def half(x, pos, dims, base):  # rotate-half: entry i paired with entry i + dims / 2
+            perm = np.concatenate([np.arange(0, dims, 2), np.arange(1, dims, 2)])
+            inv = np.argsort(perm)
+            return saved(x[..., inv], pos, dims, base)[..., perm]
+        R.rotate_pairs = half
+        assert far_from(R.forward(cfg, W, t)), "pairs"
+    finally:
+        R.rotate_pairs = saved
+    # the token's own key matters: the last row against a sequence whose last token differs
+    t2 = list(t)
+    t2[-1] = (t2[-1] + 1) % 40
+    assert row_err(rows[-1:], R.forward(cfg, W, t2)[-1:]).max() > 20 * F32_GATE
+    # the second layer with a down projection of its own (random) instead of the first layer's rows
+    c3 = copy.deepcopy(cfg)
+    del c3["layers"][1]["mixer"]["kv_from"]
+    W3 = dict(R.random_weights(c3, 32))
+    W3.update(W)
+    assert far_from(R.forward(c3, W3, t)), "kv_from"
+    W4 = dict(W)
+    W4["l1.mix.g"] = W["l1.mix.g"] * 0.0  # a gate of one half everywhere
+    assert far_from(R.forward(cfg, W4, t)), "gate"
+    s.free()
+
+
+def test_one_key_far_back_among_hundreds(backend, tmp_path):
+    """bf16 and f32 serving, 700 tokens: the query of the last positions is made to point at ONE early key (a token that occurs once), so that key carries most of the
+    weight — dropping it (another token there) moves the rows far beyond the gate, in the attention of the parallel mixer and in latent attention"""
+    for layer, dtype in ((one_layer("parallel"), "f32"), (one_layer("latent", rot_dim=0, kv_rank=24), "f32"), (one_layer("latent", rot_dim=0, kv_rank=24), "bf16")):
+        cfg = R.make_config(48, 40, [layer], side_dim=0)
+        W = R.random_weights(cfg, 33)
+        for name in list(W):
+            if name.endswith(".q") or name.endswith("mix.uq"):
+                W[name] = R.bf16_round(W[name] * 6.0)
+        if layer["type"] == "parallel":
+            W["l0.mix.right.out"] = W["l0.mix.right.out"] * 0.0
+        rng = np.random.default_rng(5)
+        t = rng.integers(0, 39, 700).tolist()
+        t[3] = 39  # occurs once
+        s = Served(backend, tmp_path / (layer["type"] + dtype), cfg, 0, dtype, W=W, max_tokens=768)
+        rows = np.concatenate([s.feed("w", t[:650])] + [s.feed("w", [x]) for x in t[650:]])
+        gate = F32_GATE if dtype == "f32" else BF16_GATE
+        ref = R.forward(cfg, W, t)
+        assert within(row_err(rows, ref), gate, dtype)
+        t2 = list(t)
+        t2[3] = 0
+        moved = row_err(ref[600:], R.forward(cfg, W, t2)[600:])
+        if dtype == "f32":
+            assert moved.max() > 20 * gate  # the reference itself says the far key matters
+            assert row_err(rows[600:], R.forward(cfg, W, t2)[600:]).max() > 20 * gate
+        s.free()
+
+
+@pytest.mark.parametrize("kind", ["ssd", "delta"])
+def test_a_token_far_back_is_carried_by_the_state(backend, tmp_path, kind):
+    """recurrences with slow decay: the first tokens of a 300-token sequence still move the last rows (the reference says so), and the engine — prompt in portions,
+    then single tokens — agrees with the reference that saw the true first tokens"""
+    layer = one_layer("ssd", state=32) if kind == "ssd" else one_layer("parallel", r_dim=64)
+    cfg = R.make_config(48, 40, [layer], side_dim=0)
+    W = R.random_weights(cfg, 35)
+    if kind == "ssd":
+        W["l0.mix.A_log"] = W["l0.mix.A_log"] * 0 - 7.0     # decay exp(-e^-7 dt): nearly none
+    else:
+        W["l0.mix.left.out"] = W["l0.mix.left.out"] * 0.0
+        W["l0.mix.right.A_log"] = W["l0.mix.right.A_log"] * 0 - 6.0
+        W["l0.mix.right.b"] = W["l0.mix.right.b"] * 0       # beta = 1/2 and 64 key entries: 300 writes leave a tenth of the first token's trace
+    s = Served(backend, tmp_path, cfg, 0, "f32", W=W)
+    t = toks(300, 40, 6)
+    rows = np.concatenate([s.feed("w", t[:100]), s.feed("w", t[100:280])] + [s.feed("w", [x]) for x in t[280:]])
+    assert row_err(rows, R.forward(cfg, W, t)).max() <= F32_GATE
+    t2 = [(x + 1) % 40 for x in t[:20]] + t[20:]
+    assert row_err(rows[290:], R.forward(cfg, W, t2)[290:]).max() > 10 * F32_GATE
+    s.free()
+
+
+def test_constants_of_the_recurrences_norms_and_side_input_show(backend, tmp_path):
+    """the engine's rows are far from the reference computed with a neighbouring constant or weight: decays, step sizes, the skip term, the convolution's bias and tap
+    order, the norm in parts, per-channel decay offsets, biases, per-head norm weights, the one-plus form of the model's norm, the side input's part of the table"""
+    cfg = R.make_config(48, 40, [one_layer("ssd", norm_groups=2, mlp=R.dense(16)), one_layer("parallel")], side_dim=6)
+    W = R.random_weights(cfg, 37)
+    s = Served(backend, tmp_path, cfg, 0, "f32", W=W)
+    t = toks(50, 40, 7)
+    rows = s.feed("w", t, end=True)
+    assert row_err(rows, R.forward(cfg, W, t)).max() <= F32_GATE
+    c2 = copy.deepcopy(cfg)
+    c2["layers"][0]["mixer"]["norm_groups"] = 1
+    assert row_err(rows, R.forward(c2, W, t)).max() > 20 * F32_GATE
+    c3 = copy.deepcopy(cfg)
+    c3["layers"][0]["mixer"]["groups"] = 1
+    W3 = dict(W)
+    W3["l0.mix.in"] = np.concatenate([W["l0.mix.in"][:32 + 32 + 12], W["l0.mix.in"][32 + 32 + 24:32 + 32 + 36], W["l0.mix.in"][-4:]])
+    W3["l0.mix.conv"] = np.concatenate([W["l0.mix.conv"][:32 + 12], W["l0.mix.conv"][32 + 24:32 + 36]])
+    W3["l0.mix.conv.b"] = np.concatenate([W["l0.mix.conv.b"][:32 + 12], W["l0.mix.conv.b"][32 + 24:32 + 36]])
+    assert row_err(rows, R.forward(c3, W3, t)).max() > 20 * F32_GATE  # (every head reading the first group)
+    for name, f in (("l0.mix.A_log", lambda a: a + 0.2), ("l0.mix.dt_bias", lambda a: a + 0.3), ("l0.mix.D", lambda a: a + 0.2), ("l0.mix.conv.b", lambda a: a + 0.1),
+                    ("l0.mix.conv", lambda a: a[:, ::-1]), ("l0.mix.norm", lambda a: a * 1.1), ("l1.mix.right.A_log", lambda a: a + 0.3),
+                    ("l1.mix.right.dt_bias", lambda a: np.roll(a, 1)), ("l1.mix.right.norm", lambda a: np.roll(a, 1)), ("l1.mix.right.v.conv", lambda a: a[:, ::-1]),
+                    ("l1.mix.left.q.norm", lambda a: np.roll(a, 1)), ("l1.mix.left.k.b", lambda a: a + 0.2), ("l1.mix.left.out", lambda a: a * 1.2),
+                    ("l1.norm1", lambda a: a - 1.0), ("l0.norm2", lambda a: a + 0.3), ("final.norm", lambda a: a - 1.0), ("l1.side.norm", lambda a: a * 1.3),
+                    ("side.embed", lambda a: np.roll(a, 6, axis=1))):
+        W2 = dict(W)
+        W2[name] = f(W[name])
+        assert row_err(rows, R.forward(cfg, W2, t)).max() > 20 * F32_GATE, name
+    s.free()
+
+
+# ------------------------------------------------------------------------------------------------ the new recurrences alone, through the C-ABI
+def _batch_layout(lens_before, lens_now, interleave):
+    """a mixed batch: sequence s has fed lens_before[s] tokens and brings lens_now[s] more.  Returns (batch row -> (seq, index in the sequence), tok, info)."""
+    order = []
+    left = list(lens_now)
+    while any(left):
+        for s in range(len(left)):
+            take = 1 if interleave else left[s]
+            for _ in range(min(take, left[s])):
+                order.append((s, lens_before[s] + lens_now[s] - left[s]))
+                left[s] -= 1
+    rows_of = {sp: i for i, sp in enumerate(order)}
+    tok, info = [], []
+    for s in range(len(lens_now)):
+        if not lens_now[s]:
+            continue
+        info.append([len(tok), lens_now[s], s, 1 if lens_before[s] == 0 else 0])
+        tok += [rows_of[(s, p)] for p in range(lens_before[s], lens_before[s] + lens_now[s])]
+    return order, np.asarray(tok, np.int32), np.asarray(info, np.int32)
+
+
+@pytest.mark.parametrize("kind,heads,kv_heads,dk,dv", [("ssd", 4, 2, 16, 8), ("ssd", 3, 1, 136, 5), ("ssd", 2, 2, 7, 33), ("ssd", 1, 1, 64, 200),
+                                                       ("delta_ch", 4, 2, 16, 8), ("delta_ch", 3, 3, 7, 12), ("delta_ch", 2, 1, 136, 40), ("delta_ch", 6, 2, 32, 64)])
+def test_recurrences_over_mixed_batches(backend, H, kind, heads, kv_heads, dk, dv):
+    """three sequences in two mixed batches against the plain token-by-token loops of the reference, the state going through the engine's own state tensor (stale values
+    in the slot of a sequence that starts)"""
+    rng = np.random.default_rng(dk * 7 + dv)
+    S = 4
+    lens = [(0, 6, 4), (0, 1, 19), (0, 0, 5)]
+    n_tok = [a + b + c for a, b, c in lens]
+    data = []
+    for n in n_tok:
+        d = dict(q=rng.standard_normal((n, kv_heads * dk)), k=rng.standard_normal((n, kv_heads * dk)), v=rng.standard_normal((n, heads * dv)),
+                 g=rng.standard_normal((n, heads * dk if kind == "delta_ch" else heads)) * 2.0, b=rng.standard_normal((n, heads)) * 2.0)
+        data.append({a: b.astype(np.float32) for a, b in d.items()})
+    if kind == "ssd":
+        p0 = np.concatenate([rng.uniform(-2.0, 0.5, heads), rng.uniform(-1.0, 1.0, heads), rng.standard_normal(heads)]).astype(np.float32)
+    else:
+        p0 = np.concatenate([rng.uniform(-2.0, 0.5, heads), rng.uniform(-1.0, 1.0, heads * dk)]).astype(np.float32)
+    size = H.ggml_seq_state_size(4 if kind == "ssd" else 3, heads, dk, dv)
+    state = np.full((S, size), 3.0, np.float32)
+    got = [np.zeros((n, heads, dv)) for n in n_tok]
+    before = [0, 0, 0]
+    for step, interleave in ((1, False), (2, True)):
+        now = [l[step] for l in lens]
+        order, tok, info = _batch_layout(before, now, interleave)
+        cat = {a: np.stack([data[s][a][p] for s, p in order]) for a in "qkvgb"}
+        g = T.G(backend)
+        t = {a: g.new(L.F32, [cat[a].shape[1], len(order)], cat[a]) for a in "qkvgb"}
+        ts = g.new(L.F32, [size, S], state)
+        tt, ti = g.new(L.I32, [len(order)], tok), g.new(L.I32, [4, len(info)], info)
+        tp = g.new(L.F32, [len(p0)], p0)
+        if kind == "ssd":
+            o = H.ggml_seq_ssd(g.ctx, t["q"], t["k"], t["v"], t["g"], tp, ts, tt, ti, heads, kv_heads)
+        else:
+            o = H.ggml_seq_delta_channel(g.ctx, t["q"], t["k"], t["v"], t["b"], t["g"], tp, ts, tt, ti, heads, kv_heads)
+        res = g.compute([o])
+        state = g.read(ts).reshape(S, size)
+        g.free()
+        y = res[0].reshape(len(order), heads, dv)
+        for i, (s, p) in enumerate(order):
+            got[s][p] = y[i]
+        before = [b + n for b, n in zip(before, now)]
+    for s, n in enumerate(n_tok):
+        d = {a: b.astype(np.float64) for a, b in data[s].items()}
+        q, k, v = d["q"].reshape(n, kv_heads, dk), d["k"].reshape(n, kv_heads, dk), d["v"].reshape(n, heads, dv)
+        if kind == "ssd":
+            dt = R.softplus(d["g"] + p0[heads:2 * heads])
+            ref = R.state_space_scan(v, k, q, dt, np.exp(p0[:heads].astype(np.float64)), p0[2 * heads:].astype(np.float64))
+        else:
+            qn = q / np.sqrt((q * q).sum(axis=-1, keepdims=True) + 1e-6) * dk ** -0.5
+            kn = k / np.sqrt((k * k).sum(axis=-1, keepdims=True) + 1e-6)
+            decay = np.exp(-np.exp(p0[:heads].astype(np.float64))[None, :, None] * R.softplus(d["g"] + p0[heads:]).reshape(n, heads, dk))
+            ref = R.delta_rule_channel_decay(qn, kn, v, R.sigmoid(d["b"]), decay)
+        assert np.abs(got[s] - ref).max() <= 2e-5 * max(1.0, np.abs(ref).max()), (s, float(np.abs(got[s] - ref).max()))
+
+
+def test_convolution_with_bias(backend, H):
+    """the short convolution with a bias before the activation, over a strided input (some columns of a wider projection), two sequences in one batch"""
+    rng = np.random.default_rng(3)
+    Cc, taps, wide = 37, 4, 50
+    x = rng.standard_normal((12, wide)).astype(np.float32)
+    w = rng.standard_normal((Cc, taps)).astype(np.float32)
+    b = rng.standard_normal(Cc).astype(np.float32)
+    order = [(0, p) for p in range(7)] + [(1, p) for p in range(5)]
+    hist = np.full((12, taps - 1), -1, np.int32)
+    for i, (s_, p) in enumerate(order):
+        for d in range(1, taps):
+            if p - d >= 0:
+                hist[i, d - 1] = i - d
+    g = T.G(backend)
+    tx = g.new(L.F32, [wide, 12], x)
+    view = H.ggml_view_2d(g.ctx, tx, Cc, 12, wide * 4, 8 * 4)
+    st = g.new(L.F32, [Cc * (taps - 1), 2], np.zeros((2, Cc * (taps - 1)), np.float32))
+    y = H.ggml_seq_conv(g.ctx, view, g.new(L.F32, [taps, Cc], w), st, g.new(L.I32, [taps - 1, 12], hist), 1)
+    H.ggml_seq_conv_set_bias(y, g.new(L.F32, [Cc], b))
+    got = g.compute([y])[0].reshape(12, Cc)
+    g.free()
+    xs = x[:, 8:8 + Cc].astype(np.float64)
+    ref = np.concatenate([R.silu(R.short_conv(xs[:7], w.astype(np.float64), b.astype(np.float64))), R.silu(R.short_conv(xs[7:], w.astype(np.float64), b.astype(np.float64)))])
+    assert np.abs(got - ref).max() <= 1e-5
+
+
+def test_trace_run_command_line(tmp_path):
+    cfg = cfg_b()
+    W = R.random_weights(cfg, 51)
+    R.save_model(cfg, W, str(tmp_path / "model"))
+    t = toks(30, cfg["vocab"], 52)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": t[:20], "want": [0, 19]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": t[20:21], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": t[21:], "want": [8]}, {"id": "b", "tokens": t[:3], "want": [2]}], "end": ["a", "b"]}]
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bin", "trace_run")
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, exe, "--model", str(tmp_path / "model"), "--dtype", "float32", "--out", str(out), "--max-tokens", "128"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    ref = R.forward(cfg, W, t)
+    r0 = np.fromfile(out / "0.f32", "<f4").reshape(-1, cfg["vocab"])
+    r2 = np.fromfile(out / "2.f32", "<f4").reshape(-1, cfg["vocab"])
+    assert not (out / "1.f32").exists()
+    assert row_err(r0, ref[[0, 19]]).max() <= F32_GATE and row_err(r2, ref[[29, 2]]).max() <= F32_GATE
+
+
+def random_config(rng):
+    layers, latent_with_rows = [], []
+    for il in range(int(rng.integers(1, 6))):
+        kind = rng.choice(["latent", "ssd", "parallel"])
+        mlp = None if rng.random() < 0.25 else R.dense(int(rng.choice([8, 12, 20, 50])))
+        if kind == "latent":
+            rot, rank, base = int(rng.choice([0, 2, 6, 16])), int(rng.choice([5, 16, 40])), float(rng.choice([50.0, 10000.0]))
+            kv_from = None
+            if latent_with_rows and rng.random() < 0.5:
+                kv_from = int(rng.choice(latent_with_rows))
+                o = layers[kv_from]["mixer"]
+                rot, rank, base = o["rot_dim"], o["kv_rank"], o["rot"]["base"]
+            else:
+                latent_with_rows.append(il)
+            layers.append(R.latent_layer(int(rng.integers(1, 6)), int(rng.choice([4, 10, 24])), rot, int(rng.choice([4, 12, 36])), rank, int(rng.choice([3, 8, 20])),
+                                         float(rng.uniform(0.1, 0.4)), mlp, base=base, kv_from=kv_from))
+        elif kind == "ssd":
+            g = int(rng.integers(1, 4))
+            h = g * int(rng.integers(1, 4))
+            vdim = int(rng.choice([4, 6, 16]))
+            ng = int(rng.choice([d for d in (1, 2, h, g) if (h * vdim) % d == 0]))
+            layers.append(R.state_space_layer(h, vdim, int(rng.choice([3, 16, 40])), g, ng, int(rng.integers(1, 6)), mlp))
+        else:
+            g, rg = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+            layers.append(R.parallel_layer(g * int(rng.integers(1, 4)), g, int(rng.choice([8, 12, 32])), int(rng.choice([8, 20, 36])), float(rng.uniform(0.1, 0.4)),
+                                           rg * int(rng.integers(1, 3)), rg, int(rng.choice([6, 16, 24])), int(rng.choice([4, 12, 40])), int(rng.integers(1, 5)), mlp,
+                                           rank=int(rng.integers(2, 9))))
+    return R.make_config(int(rng.choice([32, 44, 64])), int(rng.integers(30, 90)), layers, side_dim=int(rng.choice([0, 1, 5, 16])), eps=float(rng.choice([1e-6, 1e-5])))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations(backend, tmp_path, seed):
+    """random layer orders, sizes, taps, groups, shared rows and side sizes: a prompt portion, then portions of 1 .. 40 tokens beside a second request"""
+    rng = np.random.default_rng(1000 + seed)
+    dtype = "f32" if seed % 3 else "bf16"
+    cfg = random_config(rng)
+    s = Served(backend, tmp_path, cfg, 100 + seed, dtype, max_tokens=320)
+    a, b = toks(140, cfg["vocab"], seed), toks(60, cfg["vocab"], seed + 50)
+    got_a, got_b = [s.feed("a", a[:31])], []
+    at_a, at_b = 31, 0
+    while at_a < len(a):
+        n = int(rng.integers(1, 41))
+        entries = [{"id": "a", "tokens": a[at_a:at_a + n], "want": list(range(len(a[at_a:at_a + n])))}]
+        nb = int(rng.integers(0, 9)) if at_b < len(b) else 0
+        if nb:
+            entries.append({"id": "b", "tokens": b[at_b:at_b + nb], "want": list(range(len(b[at_b:at_b + nb])))})
+        rows = s.s.step(entries, [])
+        na = len(entries[0]["tokens"])
+        got_a.append(rows[:na])
+        if nb:
+            got_b.append(rows[na:])
+        at_a += na
+        at_b += len(entries[1]["tokens"]) if nb else 0
+    ea = row_err(np.concatenate(got_a), s.ref(a))
+    assert within(ea, s.gate, dtype), (json.dumps(cfg), int(np.argmax(ea)), float(ea.max()))
+    if got_b:
+        eb = row_err(np.concatenate(got_b), s.ref(b)[:at_b])
+        assert within(eb, s.gate, dtype) or (len(eb) < 20 and eb.max() <= 3 * s.gate), (json.dumps(cfg), int(np.argmax(eb)), float(eb.max()))
+    s.free()
