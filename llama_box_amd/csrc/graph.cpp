@@ -333,6 +333,8 @@ static ws_plan plan_ws(backend_ctx * c, const ggml_cgraph * g) {
                 p.aux_bytes = std::max(p.aux_bytes, attn_nf_mma_ws_bytes(TD(n->src[1]), fattn_mma_pick_splits(TD(n->src[1]), TD(n->src[0]))));
         } else if (n->op == GGML_OP_MUL_MAT_ID && n->src[2]) {
             p.aux_bytes = std::max(p.aux_bytes, mul_mat_id_workspace_bytes(TD(n->src[0]), TD(n->src[2])));
+        } else if (n->op == GGML_OP_GATED_LINEAR_ATTN && n->op_params[3] == MI_SEQ_OP_TAG && n->op_params[0] == SEQ_DELTA_CH && n->src[0] && n->src[3]) {
+            p.aux_bytes = std::max(p.aux_bytes, seq_recurrence_scratch_bytes(SEQ_DELTA_CH, n->op_params[1], (int) (n->src[0]->ne[0] / std::max(1, n->op_params[2])), n->src[3]->ne[1]));
         } else if (n->op == GGML_OP_FLASH_ATTN_EXT && fa_route(n) == 4) {
             continue;  // the 32-bit kernels keep their running sums on chip
         } else if (n->op == GGML_OP_FLASH_ATTN_EXT) {
@@ -2605,7 +2607,7 @@ static int run_node(exec_state & st, int i) {
             ra.cap = wkv ? 0.0f : ggml_abi_op_param_f32(n, 4);
             ra.qscale = wkv ? 1.0f : ggml_abi_op_param_f32(n, 5);
             timed_scope ts(c, "seq_recurrence", (double) info->ne[1] * (double) state->nb[1] * 2.0);
-            launch_seq_recurrence(s, kind, ra, (int) info->ne[1]);
+            launch_seq_recurrence(s, kind, ra, (int) info->ne[1], c->ws ? (char *) c->ws + st.aux_off : nullptr, c->ws && c->ws_size > st.aux_off ? c->ws_size - st.aux_off : 0);
             c->st.kernel_launches++;
             return 1;
         }

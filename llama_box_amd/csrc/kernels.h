@@ -400,12 +400,15 @@ struct seq_rec_args {
     tdesc dst;                 // [DV, H, T]
     int DK, DV, H, G;          // G: key heads (head h reads q / k head h / (H / G))
     float cap, qscale;
+    int w_ready;               // channel decay: g already holds the decays themselves (a pass of their own computed them)
 };
 
 enum { SEQ_WKV6 = 0, SEQ_DELTA = 1, SEQ_MLSTM = 2, SEQ_DELTA_CH = 3, SEQ_SSD = 4 };
 int64_t seq_recurrence_state_floats(int kind, int H, int DK, int DV);
 bool seq_recurrence_ok(int DK, int DV);
-void launch_seq_recurrence(hipStream_t s, int kind, const seq_rec_args & a, int n_seqs);
+// scratch (optional): seq_recurrence_scratch_bytes() bytes let the channel-decay kind compute a prompt portion's decays in one parallel pass
+size_t seq_recurrence_scratch_bytes(int kind, int H, int DK, int64_t T);
+void launch_seq_recurrence(hipStream_t s, int kind, const seq_rec_args & a, int n_seqs, void * scratch = nullptr, size_t scratch_bytes = 0);
 // SOFT_MAX over a router's logits, the (group-limited) descending ARGSORT of the scores, GET_ROWS of the k first and SCALE in one launch (n <= 256 experts)
 void launch_router_softmax_topk(hipStream_t s, const tdesc & logits, const tdesc & probs, const tdesc & ids, const tdesc & wts /* [1, k, T] */, int k, int groups, int keep, float wscale);
 // RMS_NORM per head -> MUL(weight: [DV] or [DV, H]) -> MUL(act(gate)), act SiLU (0) or sigmoid (1): o [DV, H, T] (rows contiguous), gate and d [DV H, T] contiguous

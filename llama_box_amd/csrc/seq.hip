@@ -109,6 +109,7 @@ constexpr int SEQ_COLS = 4;        // value columns of a wave
 constexpr int SEQ_LPC = 16;        // lanes per value column: each owns a sixteenth of the key rows
 constexpr int SEQ_NV = 32;         // registers a lane lends to the block on its way
 constexpr int SEQ_MAX_TB = 16;     // tokens of a block at most
+constexpr int SEQ_DECAY_PREPASS_MIN = 32;  // batches of this many tokens and more compute the channel decays in a pass of their own
 
 // key rows a lane owns: a sixteenth of the head's rows, rounded up to whole groups of four (its rows are neighbours, read from LDS sixteen bytes at a time)
 static inline __host__ __device__ int seq_rows_per_lane(const int DK) { return (((DK + SEQ_LPC - 1) / SEQ_LPC) + 3) / 4 * 4; }
@@ -173,7 +174,7 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
             float val = ((const float *) (base + t * nb1))[valid ? idx : 0];
             if (HAS_W) {  // the decay's offset: w0 (time mixing), or the dt_bias entries behind the heads' A_log (channel decay)
                 const float off = A.p0[(is_w && valid) ? (KIND == SEQ_DELTA_CH ? H : 0) + h * DK + fe : 0];
-                val = is_w ? val + off : val;
+                val = (is_w && !(KIND == SEQ_DELTA_CH && A.w_ready)) ? val + off : val;  // (w_ready: the operand already holds the decays themselves)
             }
             pre[i] = valid ? val : 0.0f;
             f += 64;
@@ -209,7 +210,7 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
     // channel decay: the parked raw values (projection + offset) of a block's n_tok tokens become exp(-e^A softplus(.)) — the lanes walk over the DK real entries of
     // every token only, so the softplus and the two exponentials are paid once per entry (not once per staged float)
     auto finish_decay = [&](float * dstb, const int n_tok) {
-        if (KIND == SEQ_DELTA_CH)
+        if (KIND == SEQ_DELTA_CH && !A.w_ready)
             for (int idx = lane; idx < n_tok * DK; idx += 64) {
                 const int u = idx / DK, fe = idx - u * DK;
                 float * wp = dstb + u * per_tok + off_w + fe;
@@ -237,6 +238,50 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
             fetch(rows_of[(b + 1) & 1], n_next, pre);
             if (lane < TB && b0 + 2 * TB + lane < count) row_after = A.tok[begin + b0 + 2 * TB + lane];
         }
+        if (KIND == SEQ_SSD) {
+            // the state's update waits for nothing but the state (the read-out is beside the chain), so what a token costs is the trip to LDS for its vectors: the next
+            // token's are requested before the current token's arithmetic (the delta rules and the matrix memory, whose tokens are chains of dependent reductions, gain
+            // nothing from the same: measured, and left as they are)
+            float4 nk[R / 4], nq[R / 4];
+            float nv, ng0, ng1;
+            auto stage = [&](const int u) {
+                const float * lt = cur + u * per_tok;
+                const float4 * k4 = (const float4 *) (lt + ks * RL), * q4 = (const float4 *) (lt + KP + ks * RL);
+#pragma unroll
+                for (int m = 0; m < R / 4; ++m) {
+                    nk[m] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    nq[m] = nk[m];
+                    if (EXACT || 4 * m < RL) { nk[m] = k4[m]; nq[m] = q4[m]; }
+                }
+                nv = lt[off_v + (lane >> 4)];
+                ng0 = lt[off_g];
+                ng1 = lt[off_g + 1];
+            };
+            stage(0);
+            for (int u = 0; u < n_here; ++u) {
+                float4 kk[R / 4], cq[R / 4];
+#pragma unroll
+                for (int m = 0; m < R / 4; ++m) { kk[m] = nk[m]; cq[m] = nq[m]; }
+                const float vj = nv, dtv = ng0 * vj, dec = ng1;
+                if (u + 1 < n_here) stage(u + 1);
+                float p0 = 0.0f, p1 = 0.0f, p2 = 0.0f, p3 = 0.0f;
+#pragma unroll
+                for (int m = 0; m < R / 4; ++m) {
+                    if (EXACT || 4 * m < RL) {
+                        S[4 * m] = fmaf(kk[m].x, dtv, dec * S[4 * m]);
+                        S[4 * m + 1] = fmaf(kk[m].y, dtv, dec * S[4 * m + 1]);
+                        S[4 * m + 2] = fmaf(kk[m].z, dtv, dec * S[4 * m + 2]);
+                        S[4 * m + 3] = fmaf(kk[m].w, dtv, dec * S[4 * m + 3]);
+                        p0 = fmaf(S[4 * m], cq[m].x, p0);
+                        p1 = fmaf(S[4 * m + 1], cq[m].y, p1);
+                        p2 = fmaf(S[4 * m + 2], cq[m].z, p2);
+                        p3 = fmaf(S[4 * m + 3], cq[m].w, p3);
+                    }
+                }
+                const float o = fmaf(d_skip, vj, quad_sum((p0 + p1) + (p2 + p3)));
+                if (col && ks == 0) ((float *) (A.dst.data + (int64_t) h * A.dst.nb[1] + (int64_t) trow[u] * A.dst.nb[2]))[j] = o;
+            }
+        } else
         for (int u = 0; u < n_here; ++u) {
             const float * lt = cur + u * per_tok;
             const float4 * k4 = (const float4 *) (lt + ks * RL), * q4 = (const float4 *) (lt + KP + ks * RL), * w4 = (const float4 *) (lt + off_w + ks * RL);
@@ -260,24 +305,6 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
                     }
                 }
                 o = quad_sum((p0 + p1) + (p2 + p3));
-            } else if (KIND == SEQ_SSD) {
-                const float dtv = lt[off_g] * vj, dec = lt[off_g + 1];
-                float p0 = 0.0f, p1 = 0.0f, p2 = 0.0f, p3 = 0.0f;
-#pragma unroll
-                for (int m = 0; m < R / 4; ++m) {
-                    if (EXACT || 4 * m < RL) {
-                        const float4 kk = k4[m], cq = q4[m];
-                        S[4 * m] = fmaf(kk.x, dtv, dec * S[4 * m]);
-                        S[4 * m + 1] = fmaf(kk.y, dtv, dec * S[4 * m + 1]);
-                        S[4 * m + 2] = fmaf(kk.z, dtv, dec * S[4 * m + 2]);
-                        S[4 * m + 3] = fmaf(kk.w, dtv, dec * S[4 * m + 3]);
-                        p0 = fmaf(S[4 * m], cq.x, p0);
-                        p1 = fmaf(S[4 * m + 1], cq.y, p1);
-                        p2 = fmaf(S[4 * m + 2], cq.z, p2);
-                        p3 = fmaf(S[4 * m + 3], cq.w, p3);
-                    }
-                }
-                o = fmaf(d_skip, vj, quad_sum((p0 + p1) + (p2 + p3)));
             } else if (IS_DELTA) {
                 const float beta = lt[off_g], gdec = lt[off_g + 1];
                 float kn[R], qn[R];
@@ -286,6 +313,10 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
                 for (int m = 0; m < R / 4; ++m) {
                     float4 kk = make_float4(0.f, 0.f, 0.f, 0.f), qq = kk;
                     if (EXACT || 4 * m < RL) { kk = k4[m]; qq = q4[m]; }
+                    if (KIND == SEQ_DELTA_CH && (EXACT || 4 * m < RL)) {  // one decay per key row: applied here, ahead of the unit lengths (it waits for nothing but its own load)
+                        const float4 ww = w4[m];
+                        S[4 * m] *= ww.x; S[4 * m + 1] *= ww.y; S[4 * m + 2] *= ww.z; S[4 * m + 3] *= ww.w;
+                    }
                     kn[4 * m] = kk.x; kn[4 * m + 1] = kk.y; kn[4 * m + 2] = kk.z; kn[4 * m + 3] = kk.w;
                     qn[4 * m] = qq.x; qn[4 * m + 1] = qq.y; qn[4 * m + 2] = qq.z; qn[4 * m + 3] = qq.w;
                     k2a = fmaf(kk.x, kk.x, fmaf(kk.z, kk.z, k2a));
@@ -298,10 +329,6 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
 #pragma unroll
                 for (int m = 0; m < R / 4; ++m) {
                     if (EXACT || 4 * m < RL) {
-                        if (KIND == SEQ_DELTA_CH) {  // one decay per key row
-                            const float4 ww = w4[m];
-                            S[4 * m] *= ww.x; S[4 * m + 1] *= ww.y; S[4 * m + 2] *= ww.z; S[4 * m + 3] *= ww.w;
-                        }
 #pragma unroll
                         for (int e = 0; e < 4; ++e) { kn[4 * m + e] *= kinv; if (KIND == SEQ_DELTA) S[4 * m + e] *= gdec; }
                         d0 = fmaf(S[4 * m], kn[4 * m], d0);
@@ -371,6 +398,18 @@ __global__ void __launch_bounds__(64) k_seq_recurrence(const seq_rec_args A, con
     if (KIND == SEQ_MLSTM && j0 == 0 && lane == 0) *Mm = mrun;
 }
 
+// the decays of the channel-decay delta rule for a whole batch at once, out[t][c] = exp(-exp(A_log[c / DK]) softplus(a[t][c] + dt_bias[c])) — the formula of the recurrence
+// kernel on the same values, taken out of its token-after-token loop for prompt portions (every entry is independent of every other)
+__global__ void __launch_bounds__(256) k_seq_channel_decay(const tdesc a, const float * __restrict__ p0, const int H, const int DK, float * __restrict__ out) {
+    const int64_t C = (int64_t) H * DK, t = blockIdx.y;
+    const int64_t c = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const float a_exp = expf(p0[c / DK]);
+    const float val = ((const float *) (a.data + t * a.nb[1]))[c] + p0[H + c];
+    out[t * C + c] = expf(-a_exp * seq_softplus(val));
+}
+size_t seq_recurrence_scratch_bytes(int kind, int H, int DK, int64_t T) { return (kind == SEQ_DELTA_CH && T >= SEQ_DECAY_PREPASS_MIN) ? (size_t) T * H * DK * sizeof(float) : 0; }
+
 // floats of state one slot needs
 int64_t seq_recurrence_state_floats(int kind, int H, int DK, int DV) {
     return (int64_t) H * seq_rows_per_lane(DK) * DV * SEQ_LPC + (kind == SEQ_MLSTM ? (int64_t) H * DK + H : 0);
@@ -393,8 +432,20 @@ static void seq_recurrence_launch(hipStream_t s, const seq_rec_args & a, int n_s
     else MI_SEQ_REC(16);
 #undef MI_SEQ_REC
 }
-void launch_seq_recurrence(hipStream_t s, int kind, const seq_rec_args & a, int n_seqs) {
-    if (n_seqs == 0 || a.H == 0) return;
+void launch_seq_recurrence(hipStream_t s, int kind, const seq_rec_args & a_in, int n_seqs, void * scratch, size_t scratch_bytes) {
+    if (n_seqs == 0 || a_in.H == 0) return;
+    seq_rec_args a = a_in;
+    a.w_ready = 0;
+    const int64_t T = a.g.ne[1];
+    const size_t need = seq_recurrence_scratch_bytes(kind, a.H, a.DK, T);
+    if (need > 0 && scratch && need <= scratch_bytes) {  // a prompt portion: the decays of all its tokens in one parallel pass
+        const int64_t C = (int64_t) a.H * a.DK;
+        hipLaunchKernelGGL(k_seq_channel_decay, dim3((unsigned) ((C + 255) / 256), (unsigned) T), dim3(256), 0, s, a.g, a.p0, a.H, a.DK, (float *) scratch);
+        a.g.data = (char *) scratch;
+        a.g.nb[0] = 4;
+        a.g.nb[1] = C * 4;
+        a.w_ready = 1;
+    }
     if (kind == SEQ_WKV6) seq_recurrence_launch<SEQ_WKV6>(s, a, n_seqs);
     else if (kind == SEQ_DELTA) seq_recurrence_launch<SEQ_DELTA>(s, a, n_seqs);
     else if (kind == SEQ_DELTA_CH) seq_recurrence_launch<SEQ_DELTA_CH>(s, a, n_seqs);

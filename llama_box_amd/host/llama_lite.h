@@ -63,7 +63,9 @@ struct llm_model * llm_model_load(const char * path, ggml_backend_buffer_type_t 
  * positions, a soft-max with a zero-score sink, value mixing with the first such layer, a sigmoid output gate, layer norms before and after every
  * sublayer, a dense erf-GELU or a top-k mixture-of-experts feed-forward, tied output matrix); "Zigipel" (latent and windowed attention, token shift, a
  * repeated range of layers); "Rarelorn" (mixers with state per sequence: a matrix memory with exponential gates, a gated delta rule behind short
- * convolutions, windowed sigmoid attention beside RWKV-style time mixing; experts chosen from a soft-max over all of them within the best groups).  wtype: GGML_TYPE_BF16 keeps the matrices as stored
+ * convolutions, windowed sigmoid attention beside RWKV-style time mixing; experts chosen from a soft-max over all of them within the best groups);
+ * "Nogavik" (latent attention with a query latent, optionally over an earlier layer's cache rows; a state-space mixer; attention beside a delta rule with one decay
+ * per key channel; two norms of the same input per layer; a per-layer token input; tied output matrix).  wtype: GGML_TYPE_BF16 keeps the matrices as stored
  * (bf16 products, f32 accumulation); GGML_TYPE_F32 widens them at load (everything in 32-bit).  Norm weights and routers are always f32. */
 struct llm_model * llm_model_load_dir(const char * dir, ggml_backend_buffer_type_t buft, int wtype);
 /* the same model classes from the TEXT of a config.json and seeded random weights (benchmarks at sizes no file exists for) */

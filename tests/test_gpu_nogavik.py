@@ -468,7 +468,7 @@ def test_recurrences_over_mixed_batches(backend, H, kind, heads, kv_heads, dk, d
     in the slot of a sequence that starts)"""
     rng = np.random.default_rng(dk * 7 + dv)
     S = 4
-    lens = [(0, 6, 4), (0, 1, 19), (0, 0, 5)]
+    lens = [(0, 6, 4), (0, 1, 33), (0, 0, 5)]  # (the second batch is long enough for the channel decays to take their pass of their own)
     n_tok = [a + b + c for a, b, c in lens]
     data = []
     for n in n_tok:
