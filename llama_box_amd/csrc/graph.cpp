@@ -2053,12 +2053,13 @@ static int try_fuse_gate_norm(exec_state & st, int i) {
     for (int k = 0; k < 3; ++k) mark_done(st, at[k]);
     return 1;
 }
-// RMS_NORM(l) -> MUL(wl), RMS_NORM(r) -> MUL(wr), SCALE, SCALE, ADD: two branches normed over the width and blended, one launch.  Returns the nodes consumed
+// RMS_NORM(l) -> MUL(wl) -> SCALE, RMS_NORM(r) -> MUL(wr) -> SCALE, ADD (the order in which the ADD's two operands are expanded): two branches normed over the width and
+// blended, one launch.  Returns the nodes consumed
 static int try_fuse_norm2_blend(exec_state & st, int i) {
     ggml_cgraph * g = st.g;
     if (i + 6 >= g->n_nodes) return 0;
     for (int k = 1; k <= 6; ++k) if (st.done[i + k]) return 0;
-    const ggml_tensor * n1 = g->nodes[i], * m1 = g->nodes[i + 1], * n2 = g->nodes[i + 2], * m2 = g->nodes[i + 3], * s1 = g->nodes[i + 4], * s2 = g->nodes[i + 5], * ad = g->nodes[i + 6];
+    const ggml_tensor * n1 = g->nodes[i], * m1 = g->nodes[i + 1], * s1 = g->nodes[i + 2], * n2 = g->nodes[i + 3], * m2 = g->nodes[i + 4], * s2 = g->nodes[i + 5], * ad = g->nodes[i + 6];
     if (m1->op != GGML_OP_MUL || n2->op != GGML_OP_RMS_NORM || m2->op != GGML_OP_MUL || s1->op != GGML_OP_SCALE || s2->op != GGML_OP_SCALE || ad->op != GGML_OP_ADD) return 0;
     if (m1->src[0] != n1 || m2->src[0] != n2 || s1->src[0] != m1 || s2->src[0] != m2 || ad->src[0] != s1 || ad->src[1] != s2) return 0;
     if (ggml_abi_op_param_f32(s1, 1) != 0.0f || ggml_abi_op_param_f32(s2, 1) != 0.0f || ggml_abi_op_param_f32(n1, 0) != ggml_abi_op_param_f32(n2, 0)) return 0;

@@ -507,22 +507,19 @@ void launch_add3(hipStream_t s, const float * x, const float * a, const float * 
     hipLaunchKernelGGL(k_add3, dim3((unsigned) std::min<int64_t>((n + 255) / 256, 2048)), dim3(256), 0, s, x, a, b, d, n);
 }
 // a gate in FRONT of a norm over equal parts of a row: t = y * silu(z); every part of D entries divided by its root mean square; times w (one entry per entry of the
-// row) — UNARY(SILU) -> MUL -> RMS_NORM -> MUL.  A wave per (part, token); the sum of squares in f64 as in k_rms_norm
-__global__ void __launch_bounds__(256) k_gate_norm(const float * y, const float * z, const float * __restrict__ w, float * d, const int64_t D, const int64_t parts, const int64_t rows,
-                                                   const float eps) {
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t) blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const int64_t p = row % parts;
+// row) — UNARY(SILU) -> MUL -> RMS_NORM -> MUL.  A workgroup per (part, token); the sum of squares in f64 as in k_rms_norm
+__global__ void __launch_bounds__(256) k_gate_norm(const float * y, const float * z, const float * __restrict__ w, float * d, const int64_t D, const int64_t parts, const float eps) {
+    __shared__ double sh[4];
+    const int64_t row = blockIdx.x, p = row % parts;
     const float * yr = y + row * D, * zr = z + row * D;
     double s = 0.0;
-    for (int64_t i = lane; i < D; i += 64) { const float t = yr[i] * silu_f(zr[i]); s += (double) (t * t); }
-    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) { const float t = yr[i] * silu_f(zr[i]); s += (double) (t * t); }
+    s = block_sum_d(s, sh);
     const float mean = (float) (s / (double) D);
     const float scale = 1.0f / sqrtf(mean + eps);
     const float * __restrict__ wr = w + p * D;
     float * out = d + row * D;
-    for (int64_t i = lane; i < D; i += 64) {
+    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
         const float t = yr[i] * silu_f(zr[i]);
         const float v = t * scale;
         out[i] = v * wr[i];
@@ -530,7 +527,7 @@ __global__ void __launch_bounds__(256) k_gate_norm(const float * y, const float 
 }
 void launch_gate_norm(hipStream_t s, const float * y, const float * z, const float * w, float * d, int64_t D, int64_t parts, int64_t rows, float eps) {
     if (rows == 0 || D == 0) return;
-    hipLaunchKernelGGL(k_gate_norm, dim3((unsigned) ((rows + 3) / 4)), dim3(256), 0, s, y, z, w, d, D, parts, rows, eps);
+    hipLaunchKernelGGL(k_gate_norm, dim3((unsigned) rows), dim3(256), 0, s, y, z, w, d, D, parts, eps);
 }
 // two rows normed and blended: d = a * (rms_norm(l) * wl) + b * (rms_norm(r) * wr) — RMS_NORM -> MUL, RMS_NORM -> MUL, SCALE, SCALE, ADD.  A workgroup per row; the sums
 // are taken as k_rms_norm takes them on its element-wise path

@@ -182,6 +182,15 @@ def test_graph_of_a_mixed_batch(H):
     assert rec[0][1] == "ssd-1" and rec[1][1] == "delta_channel-3" and rec[1][2][8] == "delta_b_pre-3" and rec[0][2][8] is None
     conv = [n for n in nodes if n[0] == "SSM_CONV" and not n[1].startswith("conv_store")]
     assert conv[0][2][4] == "blk.1.ssm_conv1d.bias" and conv[1][2][4] is None
+    # the two branches' norms, factors and sum follow one another (the backend runs the seven nodes as one launch)
+    names = [n[1] for n in nodes]
+    at = names.index("mix_left_rnorm-3")
+    assert names[at:at + 7] == ["mix_left_rnorm-3", "mix_left_normed-3", "mix_left-3", "mix_right_rnorm-3", "mix_right_normed-3", "mix_right-3", "mix_sum-3"]
+    # ... as do the gate's activation and its product with the side rows, and the state-space gate, its norm in parts and the weight (views between them)
+    at = names.index("side_gelu-0")
+    assert names[at + 1] == "side_gated-0"
+    at = names.index("ssm_z_silu-1")
+    assert [x for x, n in zip(names[at:at + 8], nodes[at:at + 8]) if n[0] not in ("RESHAPE", "VIEW")][:4] == ["ssm_z_silu-1", "ssm_gated-1", "ssm_rnorm-1", "ssm_normed-1"]
     # the side input: one small table per layer, read by token
     assert [n[2][0] for n in nodes if n[1].startswith("side_embd")] == ["blk.%d.side_embd.weight" % il for il in range(4)]
     # the last layer goes on with the wanted rows only: here all of them
