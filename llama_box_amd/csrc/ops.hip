@@ -507,9 +507,10 @@ void launch_add3(hipStream_t s, const float * x, const float * a, const float * 
     hipLaunchKernelGGL(k_add3, dim3((unsigned) std::min<int64_t>((n + 255) / 256, 2048)), dim3(256), 0, s, x, a, b, d, n);
 }
 // a gate in FRONT of a norm over equal parts of a row: t = y * silu(z); every part of D entries divided by its root mean square; times w (one entry per entry of the
-// row) — UNARY(SILU) -> MUL -> RMS_NORM -> MUL.  A workgroup per (part, token); the sum of squares in f64 as in k_rms_norm
-__global__ void __launch_bounds__(256) k_gate_norm(const float * y, const float * z, const float * __restrict__ w, float * d, const int64_t D, const int64_t parts, const float eps) {
-    __shared__ double sh[4];
+// row) — UNARY(SILU) -> MUL -> RMS_NORM -> MUL.  A workgroup per (part, token) — of 1024 threads for long parts: the SiLU's exponential and division are most of the work,
+// and a part of 4096 entries is one workgroup's at a decode step; the sum of squares in f64 as in k_rms_norm
+__global__ void __launch_bounds__(1024) k_gate_norm(const float * y, const float * z, const float * __restrict__ w, float * d, const int64_t D, const int64_t parts, const float eps) {
+    __shared__ double sh[16];
     const int64_t row = blockIdx.x, p = row % parts;
     const float * yr = y + row * D, * zr = z + row * D;
     double s = 0.0;
@@ -527,7 +528,7 @@ __global__ void __launch_bounds__(256) k_gate_norm(const float * y, const float 
 }
 void launch_gate_norm(hipStream_t s, const float * y, const float * z, const float * w, float * d, int64_t D, int64_t parts, int64_t rows, float eps) {
     if (rows == 0 || D == 0) return;
-    hipLaunchKernelGGL(k_gate_norm, dim3((unsigned) rows), dim3(256), 0, s, y, z, w, d, D, parts, eps);
+    hipLaunchKernelGGL(k_gate_norm, dim3((unsigned) rows), dim3(D > 1024 ? 1024 : 256), 0, s, y, z, w, d, D, parts, eps);
 }
 // two rows normed and blended: d = a * (rms_norm(l) * wl) + b * (rms_norm(r) * wr) — RMS_NORM -> MUL, RMS_NORM -> MUL, SCALE, SCALE, ADD.  A workgroup per row; the sums
 // are taken as k_rms_norm takes them on its element-wise path

@@ -86,7 +86,18 @@ def cfg_d():
     ], side_dim=24, eps=1e-6)
 
 
-CONFIGS = {"a": cfg_a, "b": cfg_b, "c": cfg_c, "d": cfg_d}
+def cfg_e():
+    # odd sizes everywhere: a width, head sizes, latents, state, taps, ff, vocabulary and side size that are multiples of nothing (rows of 37 floats are not even 8-byte
+    # multiples); one rotation pair; inner sizes of one entry
+    return R.make_config(37, 31, [
+        R.state_space_layer(heads=3, vdim=5, state=3, groups=3, norm_groups=3, conv=5, mlp=R.dense(11)),
+        R.latent_layer(heads=3, dim=5, rot_dim=2, vdim=7, kv_rank=3, q_rank=1, scale=0.4, mlp=R.dense(13), base=7.0),
+        R.parallel_layer(heads=3, kv_heads=1, dim=5, vdim=7, scale=0.4, r_heads=3, r_kv_heads=3, r_dim=3, r_vdim=5, conv=3, mlp=R.dense(9), rank=1),
+        R.latent_layer(heads=1, dim=9, rot_dim=2, vdim=3, kv_rank=3, q_rank=2, scale=0.3, mlp=None, base=7.0, kv_from=1),
+    ], side_dim=5, eps=1e-6)
+
+
+CONFIGS = {"a": cfg_a, "b": cfg_b, "c": cfg_c, "d": cfg_d, "e": cfg_e}
 
 
 class Served:
@@ -108,7 +119,7 @@ class Served:
 
 # ------------------------------------------------------------------------------------------------ whole models through the engine
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-@pytest.mark.parametrize("which", ["a", "b", "c", "d"])
+@pytest.mark.parametrize("which", ["a", "b", "c", "d", "e"])
 def test_whole_prompt(backend, tmp_path, plog, which, dtype):
     s = Served(backend, tmp_path, CONFIGS[which](), 11, dtype)
     t = toks(150, s.cfg["vocab"], 5)  # three micro-batches of 64 / 64 / 22 tokens; every position's logits
@@ -189,7 +200,7 @@ def test_prefill_against_token_by_token(backend, tmp_path, which, dtype):
     s.free()
 
 
-@pytest.mark.parametrize("which", ["a", "b", "c", "d"])
+@pytest.mark.parametrize("which", ["a", "b", "c", "d", "e"])
 def test_portions_of_every_size(backend, tmp_path, which):
     s = Served(backend, tmp_path, CONFIGS[which](), 13, "f32")
     t = toks(131, s.cfg["vocab"], 7)
