@@ -34,10 +34,10 @@ ROPE_MROPE = 8    # ggml_rope_multi: four position streams over sections of the 
 ROPE_VISION = 24  # mrope with independent sections, pairs (i, i + n_dims) over the whole row (vision towers)
 
 
-def build(verbose=False):
-    """Compile both libraries for gfx950 (hipcc cross-compiles without a GPU)."""
+def build(verbose=False, force=False):
+    """Compile both libraries for gfx950 (hipcc cross-compiles without a GPU).  force: every source is compiled again, also where its object is up to date."""
     jobs = os.environ.get("MAX_JOBS", "8")
-    r = subprocess.run(["make", "-C", _DIR, "-j" + (jobs if jobs.isdigit() else "8")], capture_output=True, text=True)
+    r = subprocess.run(["make", "-C", _DIR, "-j" + (jobs if jobs.isdigit() else "8")] + (["-B"] if force else []), capture_output=True, text=True)
     if verbose or r.returncode != 0:
         print(r.stdout[-4000:])
         print(r.stderr[-4000:])
